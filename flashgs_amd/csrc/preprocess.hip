@@ -1,0 +1,662 @@
+// Preprocess + key emission for gfx950 (wave64).
+//
+// One launch does what FlashGS preprocessCUDA (csrc/cuda_rasterizer/preprocess.cu:243-418)
+// does: near/opacity cull, projection, 2D covariance, conic, opacity-aware radius, exact
+// ellipse/tile test, (tile << 32 | depth) key emission, and - only for Gaussians that emitted a
+// key - SH colour and the 40-byte attribute record.
+//
+// Differences in mechanism (not in results):
+//  * Key slots come from a count -> wave scan -> block scan -> chained look-back over
+//    workgroups instead of atomics on one counter, so the unsorted list has a fixed order:
+//    ascending Gaussian index, then row-major tiles.  A stable sort then fixes tie order too.
+//  * Gaussians whose candidate rectangle holds at most 64 tiles test their own tiles and keep
+//    the outcome in a 64-bit mask; larger ones are tested by the whole wave, 64 tiles a step.
+//
+// THIS FILE MUST BE COMPILED WITH -ffp-contract=off.  Every fp32 expression that feeds a key is
+// written in the operand order of the reference and has to be evaluated one IEEE operation at a
+// time, so that a scalar CPU evaluation of the same expressions gives the same bits.
+#include "fgs_internal.h"
+
+#include <mutex>
+
+namespace fgs {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kSmallMax = 64;           // rectangles up to this many tiles are tested per lane
+constexpr unsigned kSpinLimit = 1u << 22;   // polls before a chained-scan wait gives up
+
+struct Camera {
+    float view[16];
+    float proj[16];
+    float campos[3];
+    int W, H, bx, by, gx, gy;
+    float tan_fovx, tan_fovy, fx, fy;
+};
+
+// ---- scalar numerics ---------------------------------------------------------------------------
+
+__device__ __forceinline__ float min_f(float a, float b) { return a < b ? a : b; }
+__device__ __forceinline__ float max_f(float a, float b) { return a > b ? a : b; }
+
+// Saturating float -> int: NaN -> 0, out-of-range clamps (the behaviour preprocess.cu:93-98 and
+// :309-310 get from the device conversion instruction).
+__device__ __forceinline__ int to_int_sat(float f)
+{
+    if (!(f == f)) return 0;
+    if (f >= 2147483648.0f) return 2147483647;
+    if (f <= -2147483648.0f) return -2147483647 - 1;
+    return (int)f;
+}
+
+// log2 of a positive normal float from its exponent plus an odd series in
+// s = (m-1)/(m+1); stands in for the approximate instruction of preprocess.cu:57-62.
+__device__ __forceinline__ float log2_det(float x)
+{
+    uint32_t bits = __float_as_uint(x);
+    int e = (int)(bits >> 23) - 127;
+    float m = __uint_as_float((bits & 0x007fffffu) | 0x3f800000u);
+    if (m > 1.41421354f) { m = m * 0.5f; e += 1; }
+    float s = (m - 1.0f) / (m + 1.0f);
+    float s2 = s * s;
+    float p = 0.111111111f;
+    p = p * s2 + 0.142857143f;
+    p = p * s2 + 0.2f;
+    p = p * s2 + 0.333333333f;
+    p = p * s2 + 1.0f;
+    float r = (s * 2.88539008f) * p;
+    return (float)e + r;
+}
+
+// preprocess.cu:64-67 - the reference's literals make this double precision.
+__device__ __forceinline__ float ndc_to_pix(float v, int S)
+{
+    return (float)((((double)v + 1.0) * (double)S - 1.0) * 0.5);
+}
+
+// 3x3 product with GLM's [col][row] storage and summation order (type_mat3x3.inl:486-519).
+struct Mat3 { float c[3][3]; };
+
+__device__ __forceinline__ Mat3 mul(const Mat3& a, const Mat3& b)
+{
+    Mat3 r;
+#pragma unroll
+    for (int col = 0; col < 3; col++)
+#pragma unroll
+        for (int row = 0; row < 3; row++)
+            r.c[col][row] = a.c[0][row] * b.c[col][0] + a.c[1][row] * b.c[col][1] + a.c[2][row] * b.c[col][2];
+    return r;
+}
+
+__device__ __forceinline__ Mat3 transposed(const Mat3& m)
+{
+    Mat3 r;
+#pragma unroll
+    for (int col = 0; col < 3; col++)
+#pragma unroll
+        for (int row = 0; row < 3; row++)
+            r.c[col][row] = m.c[row][col];
+    return r;
+}
+
+// preprocess.cu:103-143
+__device__ __forceinline__ void cov2d(const float t_in[3], const Camera& cam, const float s[6], float& c00, float& c01, float& c11)
+{
+    const float* vm = cam.view;
+    float tx = t_in[0], ty = t_in[1], tz = t_in[2];
+    const float limx = 1.3f * cam.tan_fovx;
+    const float limy = 1.3f * cam.tan_fovy;
+    const float txtz = tx / tz;
+    const float tytz = ty / tz;
+    tx = min_f(limx, max_f(-limx, txtz)) * tz;
+    ty = min_f(limy, max_f(-limy, tytz)) * tz;
+
+    Mat3 J;
+    J.c[0][0] = cam.fx / tz; J.c[0][1] = 0.0f;        J.c[0][2] = -(cam.fx * tx) / (tz * tz);
+    J.c[1][0] = 0.0f;        J.c[1][1] = cam.fy / tz; J.c[1][2] = -(cam.fy * ty) / (tz * tz);
+    J.c[2][0] = 0.0f;        J.c[2][1] = 0.0f;        J.c[2][2] = 0.0f;
+    Mat3 Wm;
+    Wm.c[0][0] = vm[0]; Wm.c[0][1] = vm[4]; Wm.c[0][2] = vm[8];
+    Wm.c[1][0] = vm[1]; Wm.c[1][1] = vm[5]; Wm.c[1][2] = vm[9];
+    Wm.c[2][0] = vm[2]; Wm.c[2][1] = vm[6]; Wm.c[2][2] = vm[10];
+    Mat3 T = mul(Wm, J);
+    Mat3 V;
+    V.c[0][0] = s[0]; V.c[0][1] = s[1]; V.c[0][2] = s[2];
+    V.c[1][0] = s[1]; V.c[1][1] = s[3]; V.c[1][2] = s[4];
+    V.c[2][0] = s[2]; V.c[2][1] = s[4]; V.c[2][2] = s[5];
+    Mat3 cov = mul(mul(transposed(T), transposed(V)), T);
+    c00 = cov.c[0][0] + 0.3f;
+    c01 = cov.c[0][1];
+    c11 = cov.c[1][1] + 0.3f;
+}
+
+// preprocess.cu:187-194
+__device__ __forceinline__ bool segment_hits(float a, float b, float c, float d, float l, float r)
+{
+    float delta = b * b - 4.0f * a * c;
+    float t1 = (l - d) * (2.0f * a) + b;
+    float t2 = (r - d) * (2.0f * a) + b;
+    return delta >= 0.0f && (t1 <= 0.0f || t1 * t1 <= delta) && (t2 >= 0.0f || t2 * t2 <= delta);
+}
+
+// preprocess.cu:238-241 || :196-236 for tile (x, y)
+__device__ __forceinline__ bool tile_hit(int x, int y, int bx, int by, float cx, float cy,
+                                         float conx, float cony, float conz, float power)
+{
+    const int minx = x * bx, miny = y * by;
+    const int maxx = minx + bx - 1, maxy = miny + by - 1;
+    const float fminx = (float)minx, fminy = (float)miny, fmaxx = (float)maxx, fmaxy = (float)maxy;
+    if (cx >= fminx && cx <= fmaxx && cy >= fminy && cy <= fmaxy) return true;
+
+    const float w = 2.0f * power;
+    float dx = (cx * 2.0f < (float)(minx + maxx)) ? cx - fminx : cx - fmaxx;
+    float a = conz;
+    float b = -2.0f * cony * dx;
+    float c = conx * dx * dx - w;
+    if (segment_hits(a, b, c, cy, fminy, fmaxy)) return true;
+
+    float dy = (cy * 2.0f < (float)(miny + maxy)) ? cy - fminy : cy - fmaxy;
+    a = conx;
+    b = -2.0f * cony * dy;
+    c = conz * dy * dy - w;
+    return segment_hits(a, b, c, cx, fminx, fmaxx);
+}
+
+// preprocess.cu:13-34, :145-185
+__device__ __forceinline__ void sh_to_rgb(const float* __restrict__ sh, float px, float py, float pz,
+                                          const Camera& cam, float rgb[3])
+{
+    constexpr float C0 = 0.28209479177387814f;
+    constexpr float C1 = 0.4886025119029199f;
+    constexpr float C2_0 = 1.0925484305920792f, C2_1 = -1.0925484305920792f, C2_2 = 0.31539156525252005f,
+                    C2_3 = -1.0925484305920792f, C2_4 = 0.5462742152960396f;
+    constexpr float C3_0 = -0.5900435899266435f, C3_1 = 2.890611442640554f, C3_2 = -0.4570457994644658f,
+                    C3_3 = 0.3731763325901154f, C3_4 = -0.4570457994644658f, C3_5 = 1.445305721320277f,
+                    C3_6 = -0.5900435899266435f;
+
+    // 48 floats = 12 aligned 16-byte loads (the record is 192 bytes)
+    float v[48];
+    const float4* src = reinterpret_cast<const float4*>(sh);
+#pragma unroll
+    for (int q = 0; q < 12; q++) {
+        float4 f = src[q];
+        v[4 * q + 0] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
+    }
+
+    float dx = px - cam.campos[0], dy = py - cam.campos[1], dz = pz - cam.campos[2];
+    float l2 = dx * dx + dy * dy + dz * dz;
+    float inv = 1.0f / __builtin_sqrtf(l2);
+    float x = dx * inv, y = dy * inv, z = dz * inv;
+    float xx = x * x, yy = y * y, zz = z * z;
+    float xy = x * y, yz = y * z, xz = x * z;
+#pragma unroll
+    for (int ch = 0; ch < 3; ch++) {
+        float res = C0 * v[ch] + 0.5f;
+        res = res - C1 * y * v[3 + ch] + C1 * z * v[6 + ch] - C1 * x * v[9 + ch];
+        res = res +
+              C2_0 * xy * v[12 + ch] +
+              C2_1 * yz * v[15 + ch] +
+              C2_2 * (2.0f * zz - xx - yy) * v[18 + ch] +
+              C2_3 * xz * v[21 + ch] +
+              C2_4 * (xx - yy) * v[24 + ch];
+        res = res +
+              C3_0 * y * (3.0f * xx - yy) * v[27 + ch] +
+              C3_1 * xy * z * v[30 + ch] +
+              C3_2 * y * (4.0f * zz - xx - yy) * v[33 + ch] +
+              C3_3 * z * (2.0f * zz - 3.0f * xx - 3.0f * yy) * v[36 + ch] +
+              C3_4 * x * (4.0f * zz - xx - yy) * v[39 + ch] +
+              C3_5 * z * (xx - yy) * v[42 + ch] +
+              C3_6 * x * (xx - 3.0f * yy) * v[45 + ch];
+        rgb[ch] = max_f(res, 0.0f);
+    }
+}
+
+// ---- chained scan over workgroups ---------------------------------------------------------------
+//
+// status word: [63:34] epoch of the launch, [33:32] state, [31:0] count.
+// A word whose epoch differs from the running launch's reads as "nothing published yet", so the
+// array never has to be cleared between launches.
+constexpr uint64_t kStateAggregate = 1;   // count of this workgroup only
+constexpr uint64_t kStatePrefix = 2;      // count of this workgroup and all before it
+constexpr uint64_t kStatePoison = 3;      // like kStatePrefix, but a predecessor never published
+
+__device__ __forceinline__ uint64_t pack_status(uint32_t epoch, uint64_t state, uint32_t value)
+{
+    return ((uint64_t)epoch << 34) | (state << 32) | (uint64_t)value;
+}
+
+__device__ __forceinline__ void publish(uint64_t* slot, uint64_t word)
+{
+    __hip_atomic_store(slot, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ uint64_t peek(const uint64_t* slot)
+{
+    return __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Executed by the first wave of a workgroup with ticket > 0.  Lane l inspects the workgroup
+// `top - l`; the walk ends at the nearest one that has published a prefix.  Returns the sum of
+// the key counts of all workgroups with a smaller ticket.  *failed is set when a predecessor
+// stayed silent for kSpinLimit polls or reported such a failure itself; the wait is bounded so
+// that every wave of the grid exits whatever happens.
+__device__ __forceinline__ uint32_t look_back(const uint64_t* status, int ticket, uint32_t epoch, bool* failed)
+{
+    const int lane = lane_id();
+    uint32_t sum = 0;
+    unsigned spins = 0;
+    int top = ticket - 1;
+    for (;;) {
+        const int j = top - lane;
+        uint64_t w = 0;
+        uint32_t state = 0;
+        uint64_t closing = 0;        // lanes holding a prefix (or poison) word
+        for (;;) {
+            state = 0;
+            if (j >= 0) {
+                w = peek(status + j);
+                if ((uint32_t)(w >> 34) == epoch) state = (uint32_t)(w >> 32) & 3u;
+            }
+            const uint64_t pending = ballot(j >= 0 && state == 0);
+            closing = ballot(state >= kStatePrefix);
+            const uint64_t need = closing ? ((closing & (~closing + 1)) << 1) - 1 : ~0ull;
+            if ((pending & need) == 0) break;
+            if (++spins > kSpinLimit) { *failed = true; return sum; }
+            __builtin_amdgcn_s_sleep(2);
+        }
+        const uint64_t first = closing & (~closing + 1);
+        const uint64_t take = closing ? (first << 1) - 1 : ~0ull;
+        if (ballot(state == kStatePoison) & first) *failed = true;
+        uint32_t v = (j >= 0 && ((take >> lane) & 1)) ? (uint32_t)w : 0u;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v += (uint32_t)__shfl_xor((int)v, o);
+        sum += v;
+        if (closing || top - kWave < 0) return sum;
+        top -= kWave;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void preprocess_kernel(
+    int P,
+    const float* __restrict__ positions,
+    const float* __restrict__ shs,
+    const float* __restrict__ opacities,
+    const float* __restrict__ cov3ds,
+    Camera cam,
+    float* __restrict__ points_xy,
+    float* __restrict__ rgb_depth,
+    float* __restrict__ conic_opacity,
+    uint64_t* __restrict__ keys,
+    uint32_t* __restrict__ values,
+    int* __restrict__ curr_offset,
+    int64_t capacity,            // <= 0: unchecked
+    uint64_t* __restrict__ status,
+    uint32_t* __restrict__ ticket_counter,
+    uint32_t ticket_base,
+    uint32_t epoch,
+    int num_blocks)
+{
+    __shared__ int s_ticket;
+    __shared__ uint32_t s_wave_total[kWavesPerBlock];
+    __shared__ uint32_t s_block_base;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+
+    if (tid == 0) s_ticket = (int)(atomicAdd(ticket_counter, 1u) - ticket_base);
+    __syncthreads();
+    const int ticket = s_ticket;
+    const int idx = ticket * kBlock + tid;
+
+    // ---- per-Gaussian state (preprocess.cu:282-316) ----
+    bool cand = false;           // passed both culls and has a non-empty candidate rectangle
+    float px = 0.f, py = 0.f, pz = 0.f;
+    float depth = 0.f;
+    float cx = 0.f, cy = 0.f;
+    float conx = 0.f, cony = 0.f, conz = 0.f;
+    float power = 0.f, log2_op = 0.f;
+    int rminx = 0, rminy = 0, rw = 0, rh = 0;
+
+    if (idx < P) {
+        px = positions[3 * (size_t)idx + 0];
+        py = positions[3 * (size_t)idx + 1];
+        pz = positions[3 * (size_t)idx + 2];
+        const float* m = cam.view;
+        float t[3];
+        t[0] = m[0] * px + m[4] * py + m[8] * pz + m[12];
+        t[1] = m[1] * px + m[5] * py + m[9] * pz + m[13];
+        t[2] = m[2] * px + m[6] * py + m[10] * pz + m[14];
+        depth = t[2];
+        if (t[2] > 0.2f) {
+            const float opacity = opacities[idx];
+            if (!(255.0f * opacity < 1.0f)) {
+                const float* q = cam.proj;
+                float hx = q[0] * px + q[4] * py + q[8] * pz + q[12];
+                float hy = q[1] * px + q[5] * py + q[9] * pz + q[13];
+                float hw = q[3] * px + q[7] * py + q[11] * pz + q[15];
+                float p_w = 1.0f / (hw + 0.0000001f);
+                float projx = hx * p_w, projy = hy * p_w;
+
+                float s[6];
+                const float2* cv = reinterpret_cast<const float2*>(cov3ds + 6 * (size_t)idx);
+                float2 s01 = cv[0], s23 = cv[1], s45 = cv[2];
+                s[0] = s01.x; s[1] = s01.y; s[2] = s23.x; s[3] = s23.y; s[4] = s45.x; s[5] = s45.y;
+                float c00, c01, c11;
+                cov2d(t, cam, s, c00, c01, c11);
+
+                float det = c00 * c11 - c01 * c01;
+                float det_inv = 1.0f / det;
+                conx = c11 * det_inv;
+                cony = -c01 * det_inv;
+                conz = c00 * det_inv;
+
+                log2_op = log2_det(opacity);
+                power = 0.69314718055f * 8.0f + 0.69314718055f * log2_op;
+                int ext_x = to_int_sat(1.414214f * __builtin_sqrtf(c00 * power) + 1.0f);
+                int ext_y = to_int_sat(1.414214f * __builtin_sqrtf(c11 * power) + 1.0f);
+
+                cx = ndc_to_pix(projx, cam.W);
+                cy = ndc_to_pix(projy, cam.H);
+                // preprocess.cu:90-100
+                rminx = min(cam.gx, max(0, to_int_sat((cx - (float)ext_x) / (float)cam.bx)));
+                rminy = min(cam.gy, max(0, to_int_sat((cy - (float)ext_y) / (float)cam.by)));
+                int rmaxx = min(cam.gx, max(0, to_int_sat((cx + (float)ext_x) / (float)cam.bx) + 1));
+                int rmaxy = min(cam.gy, max(0, to_int_sat((cy + (float)ext_y) / (float)cam.by) + 1));
+                rw = rmaxx - rminx;
+                rh = rmaxy - rminy;
+                cand = rw * rh > 0;
+            }
+        }
+    }
+    // a rectangle with both extents negative has a positive product but no tiles
+    const bool has_tiles = cand && rw > 0;
+    const int area = has_tiles ? rw * rh : 0;
+    const bool small = has_tiles && area <= kSmallMax;
+    const bool large = has_tiles && area > kSmallMax;
+
+    // ---- count keys ----
+    uint64_t hit_mask = 0;
+    uint32_t count = 0;
+    if (small) {
+        int x = rminx, y = rminy;
+        for (int j = 0; j < area; j++) {
+            if (tile_hit(x, y, cam.bx, cam.by, cx, cy, conx, cony, conz, power)) hit_mask |= 1ull << j;
+            if (++x == rminx + rw) { x = rminx; y++; }
+        }
+        count = (uint32_t)__popcll(hit_mask);
+    }
+    const uint64_t large_lanes = ballot(large);
+    for (uint64_t todo = large_lanes; todo; todo &= todo - 1) {
+        const int src = __ffsll((long long)todo) - 1;
+        const float gcx = bcast_f(cx, src), gcy = bcast_f(cy, src);
+        const float gconx = bcast_f(conx, src), gcony = bcast_f(cony, src), gconz = bcast_f(conz, src);
+        const float gpower = bcast_f(power, src);
+        const int gminx = bcast_i(rminx, src), gminy = bcast_i(rminy, src);
+        const int grw = bcast_i(rw, src), garea = bcast_i(area, src);
+        uint32_t total = 0;
+        for (int base = 0; base < garea; base += kWave) {
+            const int j = base + lane;
+            bool ok = false;
+            if (j < garea) {
+                const int ty = j / grw, tx = j - ty * grw;
+                ok = tile_hit(gminx + tx, gminy + ty, cam.bx, cam.by, gcx, gcy, gconx, gcony, gconz, gpower);
+            }
+            total += (uint32_t)__popcll(ballot(ok));
+        }
+        if (lane == src) count = total;
+    }
+
+    // ---- slots: wave scan, block scan, chained scan over workgroups ----
+    uint32_t incl = count;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        uint32_t up = (uint32_t)__shfl_up((int)incl, o);
+        if (lane >= o) incl += up;
+    }
+    const uint32_t wave_total = (uint32_t)bcast_i((int)incl, kWave - 1);
+    if (lane == 0) s_wave_total[wave] = wave_total;
+    __syncthreads();
+
+    uint32_t wave_base = 0, block_total = 0;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; w++) {
+        uint32_t t = s_wave_total[w];
+        if (w < wave) wave_base += t;
+        block_total += t;
+    }
+
+    if (wave == 0) {
+        bool timed_out = false;
+        uint32_t excl;
+        if (ticket == 0) {
+            excl = (uint32_t)*curr_offset;     // the caller's starting offset (example.py:69 zeroes it)
+        } else {
+            if (lane == 0) publish(status + ticket, pack_status(epoch, kStateAggregate, block_total));
+            excl = look_back(status, ticket, epoch, &timed_out);
+        }
+        if (lane == 0) {
+            publish(status + ticket, pack_status(epoch, timed_out ? kStatePoison : kStatePrefix, excl + block_total));
+            s_block_base = excl;
+            // only the last workgroup writes the counter; a poisoned chain yields a negative count
+            if (ticket == num_blocks - 1) *curr_offset = timed_out ? -2147483647 - 1 : (int)(excl + block_total);
+        }
+    }
+    __syncthreads();
+    const uint32_t my_slot = s_block_base + wave_base + (incl - count);
+
+    // ---- emit ----
+    const uint64_t cap = capacity > 0 ? (uint64_t)capacity : ~0ull;
+    const uint32_t depth_bits = __float_as_uint(depth);
+    if (small && hit_mask) {
+        uint64_t slot = my_slot;
+        int x = rminx, y = rminy;
+        for (int j = 0; j < area; j++) {
+            if ((hit_mask >> j) & 1) {
+                if (slot < cap) {
+                    keys[slot] = ((uint64_t)(uint32_t)(y * cam.gx + x) << 32) | depth_bits;
+                    values[slot] = (uint32_t)idx;
+                }
+                slot++;
+            }
+            if (++x == rminx + rw) { x = rminx; y++; }
+        }
+    }
+    for (uint64_t todo = large_lanes; todo; todo &= todo - 1) {
+        const int src = __ffsll((long long)todo) - 1;
+        if (bcast_i((int)count, src) == 0) continue;
+        const float gcx = bcast_f(cx, src), gcy = bcast_f(cy, src);
+        const float gconx = bcast_f(conx, src), gcony = bcast_f(cony, src), gconz = bcast_f(conz, src);
+        const float gpower = bcast_f(power, src);
+        const int gminx = bcast_i(rminx, src), gminy = bcast_i(rminy, src);
+        const int grw = bcast_i(rw, src), garea = bcast_i(area, src);
+        const uint32_t gdepth = (uint32_t)bcast_i((int)depth_bits, src);
+        const uint32_t gidx = (uint32_t)(ticket * kBlock + wave * kWave + src);
+        uint64_t slot = (uint32_t)bcast_i((int)my_slot, src);
+        for (int base = 0; base < garea; base += kWave) {
+            const int j = base + lane;
+            bool ok = false;
+            int tx = 0, ty = 0;
+            if (j < garea) {
+                ty = j / grw; tx = j - ty * grw;
+                ok = tile_hit(gminx + tx, gminy + ty, cam.bx, cam.by, gcx, gcy, gconx, gcony, gconz, gpower);
+            }
+            const uint64_t hits = ballot(ok);
+            if (ok) {
+                const uint64_t dst = slot + (uint64_t)popc_below(hits);
+                if (dst < cap) {
+                    keys[dst] = ((uint64_t)(uint32_t)((gminy + ty) * cam.gx + gminx + tx) << 32) | gdepth;
+                    values[dst] = gidx;
+                }
+            }
+            slot += (uint64_t)__popcll(hits);
+        }
+    }
+
+    // ---- attributes of Gaussians that emitted a key (preprocess.cu:411-417) ----
+    if (count > 0) {
+        constexpr float log2e = 1.4426950216293334961f;
+        reinterpret_cast<float2*>(points_xy)[idx] = make_float2(cx, cy);
+        reinterpret_cast<float4*>(conic_opacity)[idx] =
+            make_float4((-0.5f * log2e) * conx, -log2e * cony, (-0.5f * log2e) * conz, log2_op);
+        float rgb[3];
+        sh_to_rgb(shs + 48 * (size_t)idx, px, py, pz, cam, rgb);
+        reinterpret_cast<float4*>(rgb_depth)[idx] = make_float4(rgb[0], rgb[1], rgb[2], depth);
+    }
+}
+
+// ---- per-device scratch for the chained scan ------------------------------------------------------
+
+struct Scratch {
+    uint64_t* status = nullptr;     // one word per workgroup
+    size_t status_words = 0;
+    uint32_t* ticket = nullptr;     // monotonically increasing ticket counter
+    uint32_t tickets_issued = 0;    // host mirror of *ticket (mod 2^32)
+    uint32_t epoch = 0;
+};
+
+constexpr int kMaxDevices = 64;
+Scratch g_scratch[kMaxDevices];
+std::mutex g_mutex;
+
+int acquire_scratch(int device, int num_blocks, hipStream_t stream, Scratch** out)
+{
+    Scratch& s = g_scratch[device];
+    if (s.ticket == nullptr) {
+        FGS_HIP_TRY(hipMalloc((void**)&s.ticket, 256));
+        FGS_HIP_TRY(hipMemset(s.ticket, 0, 256));
+        FGS_HIP_TRY(hipDeviceSynchronize());
+        s.tickets_issued = 0;
+    }
+    if (s.status_words < (size_t)num_blocks) {
+        // the stream may still be reading the old array: drain it before the swap
+        FGS_HIP_TRY(hipStreamSynchronize(stream));
+        if (s.status) FGS_HIP_TRY(hipFree(s.status));
+        s.status = nullptr;
+        s.status_words = 0;
+        size_t words = 1;
+        while (words < (size_t)num_blocks) words <<= 1;
+        if (words < 4096) words = 4096;
+        if (hipMalloc((void**)&s.status, words * sizeof(uint64_t)) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(FGS_E_NOMEM, "cannot allocate %zu bytes of scan status", words * sizeof(uint64_t));
+        }
+        FGS_HIP_TRY(hipMemset(s.status, 0, words * sizeof(uint64_t)));
+        FGS_HIP_TRY(hipDeviceSynchronize());
+        s.status_words = words;
+        s.epoch = 0;
+    }
+    if (s.epoch >= (1u << 30) - 1) {   // epoch field is 30 bits wide: start over on a clean array
+        FGS_HIP_TRY(hipStreamSynchronize(stream));
+        FGS_HIP_TRY(hipMemset(s.status, 0, s.status_words * sizeof(uint64_t)));
+        FGS_HIP_TRY(hipDeviceSynchronize());
+        s.epoch = 0;
+    }
+    s.epoch++;
+    *out = &s;
+    return FGS_OK;
+}
+
+} // namespace
+
+void camera_matrices(const float pos[3], const float rot[9], int width, int height,
+                     float fx, float fy, float zFar, float zNear, float view[16], float proj[16])
+{
+    // View matrix (preprocess.cu:420-427).  The nine rotation floats fill GLM columns
+    // (pybind.cpp:140-143), so column c of the upper 3x3 is rot[3c..3c+2]; the translation column
+    // is rotation * (-position) with GLM's mat3 * vec3 order (type_mat3x3.inl:468-474).
+    const float nx = -pos[0], ny = -pos[1], nz = -pos[2];
+    for (int c = 0; c < 3; c++) {
+        view[4 * c + 0] = rot[3 * c + 0];
+        view[4 * c + 1] = rot[3 * c + 1];
+        view[4 * c + 2] = rot[3 * c + 2];
+        view[4 * c + 3] = 0.0f;
+    }
+    for (int r = 0; r < 3; r++) view[12 + r] = rot[r] * nx + rot[3 + r] * ny + rot[6 + r] * nz;
+    view[15] = 1.0f;
+
+    // Projection (preprocess.cu:429-448): proj = transpose(P) * view, GLM mat4 product order
+    // (type_mat4x4.inl:630-648).  A[c][r] below is transpose(P) in [col][row] storage.
+    const float top = (float)height / (2.0f * fy) * zNear;
+    const float bottom = -top;
+    const float right = (float)width / (2.0f * fx) * zNear;
+    const float left = -right;
+    float A[4][4] = {};
+    A[0][0] = 2.0f * zNear / (right - left);
+    A[1][1] = 2.0f * zNear / (top - bottom);
+    A[2][0] = (right + left) / (right - left);
+    A[2][1] = (top + bottom) / (top - bottom);
+    A[2][3] = 1.0f;
+    A[2][2] = 1.0f * zFar / (zFar - zNear);
+    A[3][2] = -(zFar * zNear) / (zFar - zNear);
+    for (int c = 0; c < 4; c++)
+        for (int r = 0; r < 4; r++)
+            proj[4 * c + r] = A[0][r] * view[4 * c + 0] + A[1][r] * view[4 * c + 1] +
+                              A[2][r] * view[4 * c + 2] + A[3][r] * view[4 * c + 3];
+}
+
+} // namespace fgs
+
+extern "C" void fgs_camera_matrices(const float cam_position[3], const float cam_rotation[9],
+                                    int width, int height, float focal_x, float focal_y, float zFar, float zNear,
+                                    float view[16], float proj[16])
+{
+    fgs::camera_matrices(cam_position, cam_rotation, width, height, focal_x, focal_y, zFar, zNear, view, proj);
+}
+
+extern "C" int fgs_preprocess(int P,
+                              const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
+                              int width, int height, int block_x, int block_y,
+                              const float cam_position[3], const float cam_rotation[9],
+                              float focal_x, float focal_y, float zFar, float zNear,
+                              float* points_xy, float* rgb_depth, float* conic_opacity,
+                              uint64_t* gaussian_keys_unsorted, uint32_t* gaussian_values_unsorted,
+                              int* curr_offset, int64_t key_capacity, void* stream)
+{
+    using namespace fgs;
+    if (P < 0) return fail(FGS_E_INVALID, "fgs_preprocess: P = %d is negative", P);
+    if (width <= 0 || height <= 0 || block_x <= 0 || block_y <= 0)
+        return fail(FGS_E_INVALID, "fgs_preprocess: width/height/block must be positive (got %d x %d, block %d x %d)",
+                    width, height, block_x, block_y);
+    if (!cam_position || !cam_rotation) return fail(FGS_E_INVALID, "fgs_preprocess: null camera");
+    if (!curr_offset) return fail(FGS_E_INVALID, "fgs_preprocess: null curr_offset");
+    if (P > 0 && (!positions || !shs || !opacities || !cov3Ds || !points_xy || !rgb_depth || !conic_opacity ||
+                  !gaussian_keys_unsorted || !gaussian_values_unsorted))
+        return fail(FGS_E_INVALID, "fgs_preprocess: null buffer");
+    if (P == 0) return FGS_OK;
+    if (((uintptr_t)shs | (uintptr_t)rgb_depth | (uintptr_t)conic_opacity) % 16 != 0 ||
+        ((uintptr_t)cov3Ds | (uintptr_t)points_xy | (uintptr_t)gaussian_keys_unsorted) % 8 != 0)
+        return fail(FGS_E_INVALID, "fgs_preprocess: shs/rgb_depth/conic_opacity must be 16-byte aligned, "
+                                   "cov3Ds/points_xy/keys 8-byte aligned");
+    if ((long long)P + kBlock > 2147483647LL) return fail(FGS_E_INVALID, "fgs_preprocess: P = %d too large", P);
+
+    Camera cam;
+    camera_matrices(cam_position, cam_rotation, width, height, focal_x, focal_y, zFar, zNear, cam.view, cam.proj);
+    cam.campos[0] = cam_position[0]; cam.campos[1] = cam_position[1]; cam.campos[2] = cam_position[2];
+    cam.W = width; cam.H = height; cam.bx = block_x; cam.by = block_y;
+    cam.gx = (width + block_x - 1) / block_x;      // preprocess.cu:461
+    cam.gy = (height + block_y - 1) / block_y;
+    cam.tan_fovx = (float)width / (2.0f * focal_x);   // preprocess.cu:465-466
+    cam.tan_fovy = (float)height / (2.0f * focal_y);
+    cam.fx = focal_x; cam.fy = focal_y;
+
+    int device = 0;
+    FGS_HIP_TRY(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return fail(FGS_E_INVALID, "fgs_preprocess: device %d unsupported", device);
+    const int num_blocks = (P + kBlock - 1) / kBlock;
+    hipStream_t st = (hipStream_t)stream;
+
+    std::lock_guard<std::mutex> lock(g_mutex);
+    Scratch* s = nullptr;
+    int rc = acquire_scratch(device, num_blocks, st, &s);
+    if (rc != FGS_OK) return rc;
+    const uint32_t ticket_base = s->tickets_issued;
+    s->tickets_issued += (uint32_t)num_blocks;
+
+    hipLaunchKernelGGL(preprocess_kernel, dim3(num_blocks), dim3(kBlock), 0, st,
+                       P, positions, shs, opacities, cov3Ds, cam, points_xy, rgb_depth, conic_opacity,
+                       gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset, key_capacity,
+                       s->status, s->ticket, ticket_base, s->epoch, num_blocks);
+    return check_hip(hipGetLastError(), "preprocess_kernel launch");
+}

@@ -1,0 +1,125 @@
+/*
+ * flashgs_hip.h - C ABI of the MI355X (gfx950) 3D Gaussian Splatting forward rasterizer.
+ *
+ * One entry point per host function of FlashGS's csrc/ops.h:32-65; each comment cites the
+ * reference interface it replaces (paths relative to the FlashGS source tree).  Everything is
+ * plain pointers and sizes: device pointers are raw HIP device addresses, `stream` is a
+ * hipStream_t passed as void* (NULL = the default stream), cameras and colours are host
+ * arrays.  All buffers are caller-owned; calls are asynchronous on `stream` and never
+ * synchronise.  Every function that can fail returns 0 on success or a negative FGS_E_* code,
+ * with a per-thread message available from fgs_last_error().
+ */
+#ifndef FLASHGS_HIP_H
+#define FLASHGS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FGS_OK            0
+#define FGS_E_INVALID    -1   /* null pointer, negative size, unsupported tile size */
+#define FGS_E_WORKSPACE  -2   /* list_sorting_space too small for num_rendered */
+#define FGS_E_HIP        -3   /* a HIP runtime call or kernel launch failed */
+#define FGS_E_NOMEM      -4   /* internal scratch allocation failed */
+
+/* Largest key count the sort accepts (status words carry 30-bit counts). */
+#define FGS_MAX_RENDERED ((1 << 30) - 1)
+
+/*
+ * Replaces flashgs::preprocess (csrc/ops.h:32-39, csrc/cuda_rasterizer/preprocess.cu:452-488).
+ * Same arguments in the same order, with the camera as host arrays: cam_position[3] and
+ * cam_rotation[9] exactly as csrc/pybind.cpp:131-143 reads them from the two CPU tensors
+ * (cam_rotation[3*c + r] becomes element r of GLM column c).
+ *
+ * positions f32[P,3], shs f32[P,48], opacities f32[P], cov3Ds f32[P,6] are device inputs;
+ * points_xy f32[P,2], rgb_depth f32[P,4], conic_opacity f32[P,4] are device outputs whose rows
+ * are written only for Gaussians that emit at least one key; keys/values receive the
+ * (tile << 32 | depth bits, Gaussian index) pairs starting at *curr_offset, in ascending
+ * Gaussian index then row-major tile order; *curr_offset (device int, zeroed by the caller as
+ * in example.py:69) ends at the total number of pairs.
+ *
+ * key_capacity is the one addition to the reference signature: number of elements the key and
+ * value buffers hold.  Pairs that would land at or beyond it are dropped (the counter still
+ * counts them, so the caller's check of example.py:79-82 keeps working); pass 0 to write
+ * unchecked like the reference (preprocess.cu:330,395).
+ */
+int fgs_preprocess(int P,
+                   const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
+                   int width, int height, int block_x, int block_y,
+                   const float cam_position[3], const float cam_rotation[9],
+                   float focal_x, float focal_y, float zFar, float zNear,
+                   float* points_xy, float* rgb_depth, float* conic_opacity,
+                   uint64_t* gaussian_keys_unsorted, uint32_t* gaussian_values_unsorted,
+                   int* curr_offset, int64_t key_capacity, void* stream);
+
+/*
+ * Replaces flashgs::sort_gaussian (csrc/ops.h:41-45, csrc/cuda_rasterizer/sort.cu:28-44):
+ * stable ascending sort of num_rendered (key, value) pairs on key bits
+ * [0, 32 + bit_length(tiles_x * tiles_y)).  Inputs are left untouched.
+ * list_sorting_space must hold at least fgs_get_sort_buffer_size(num_rendered) bytes and be
+ * 256-byte aligned.
+ */
+int fgs_sort_gaussian(int num_rendered,
+                      int width, int height, int block_x, int block_y,
+                      char* list_sorting_space, size_t sorting_size,
+                      const uint64_t* gaussian_keys_unsorted, const uint32_t* gaussian_values_unsorted,
+                      uint64_t* gaussian_keys_sorted, uint32_t* gaussian_values_sorted, void* stream);
+
+/*
+ * Replaces flashgs::get_sort_buffer_size (csrc/ops.h:47, sort.cu:46-54).  Host only.
+ * Monotonic in num_rendered; returns 0 for a negative or too large count.
+ */
+size_t fgs_get_sort_buffer_size(int num_rendered);
+
+/*
+ * Replace flashgs::render_16x16 / render_32x16 / render_32x32 (csrc/ops.h:49-65,
+ * csrc/cuda_rasterizer/render.cu:549-608): zero `ranges`, find each tile's [start,end) in the
+ * sorted keys, blend front to back and write out_color u8[H,W,3].  `ranges` int32[tiles,2] is
+ * scratch that holds the tile ranges afterwards.  bg_color is a host array of 3 floats.
+ */
+int fgs_render_16x16(int num_rendered, int width, int height,
+                     const float* points_xy, const float* rgb_depth, const float* conic_opacity,
+                     const uint64_t* gaussian_keys_sorted, const uint32_t* gaussian_values_sorted,
+                     int* ranges, const float bg_color[3], uint8_t* out_color, void* stream);
+int fgs_render_32x16(int num_rendered, int width, int height,
+                     const float* points_xy, const float* rgb_depth, const float* conic_opacity,
+                     const uint64_t* gaussian_keys_sorted, const uint32_t* gaussian_values_sorted,
+                     int* ranges, const float bg_color[3], uint8_t* out_color, void* stream);
+int fgs_render_32x32(int num_rendered, int width, int height,
+                     const float* points_xy, const float* rgb_depth, const float* conic_opacity,
+                     const uint64_t* gaussian_keys_sorted, const uint32_t* gaussian_values_sorted,
+                     int* ranges, const float bg_color[3], uint8_t* out_color, void* stream);
+
+/*
+ * No counterpart in the reference: the same pass as fgs_render_<bx>x<by> with the colour
+ * C + T*bg stored as f32[H,W,3] before the truncating 8-bit encode of render.cu:54-57, so that
+ * images can be compared below one 8-bit step.  out_color_u8 may be NULL.
+ * block_x x block_y must be 16x16, 32x16 or 32x32.
+ */
+int fgs_render_f32(int block_x, int block_y, int num_rendered, int width, int height,
+                   const float* points_xy, const float* rgb_depth, const float* conic_opacity,
+                   const uint64_t* gaussian_keys_sorted, const uint32_t* gaussian_values_sorted,
+                   int* ranges, const float bg_color[3], uint8_t* out_color_u8, float* out_color_f32,
+                   void* stream);
+
+/*
+ * Host-side camera set-up used by fgs_preprocess (preprocess.cu:420-448,461-466), exposed so
+ * callers and tests can inspect it: column-major 4x4 view and projection matrices.
+ */
+void fgs_camera_matrices(const float cam_position[3], const float cam_rotation[9],
+                         int width, int height, float focal_x, float focal_y, float zFar, float zNear,
+                         float view[16], float proj[16]);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* fgs_last_error(void);
+
+/* ABI version of this header: bumped when a signature changes. */
+int fgs_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHGS_HIP_H */
