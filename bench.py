@@ -1,0 +1,226 @@
+#!/usr/bin/env python3
+"""Frame-rate benchmark of the forward rasterizer on one MI355X.
+
+A step is one full frame of the FlashGS forward sequence (``example.py:67-94`` of the reference):
+zero the pair counter, preprocess + key emission, the blocking 4-byte read of the pair count, radix
+sort, tile ranges, blend - on a synthetic scene that is resident in HBM before timing starts.  All
+calls go through the C ABI of libflashgs_hip.so on torch's current HIP stream; the output image
+and every work buffer are allocated once, outside the timed region.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..4] [--no-cpu-baseline]
+
+Prints one JSON line.  ``value`` is frames per second of the whole frame; ``roofline`` describes
+the dominant kernel (the blend), ``stages`` every stage with its algorithmic bytes against the
+8 TB/s HBM peak, ``cpu_baseline`` the same frame computed by the multithreaded CPU oracle on this
+machine's host cores.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
+FP32_PEAK_TFLOPS = 157.3         # MI355X fp32 vector, published (packed FMA)
+LANE_SLOTS_PER_S = 256 * 4 * 16 * 2.4e9   # VALU issue slots per second without packed math
+FLOP_PER_EVAL = 19               # render.cu:40-52: 2 sub, 6 mul + 3 add, 1 mul, 3 FMA, 1 sub
+SLOTS_PER_EVAL = 17              # 13 VALU with FMA contraction + a quarter-rate exp2
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (default: the 4K / 3M headline)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-reps", type=int, default=3)
+    return ap.parse_args()
+
+
+def cpu_baseline(sc, cam, capacity, reps):
+    """The CPU oracle (a port of the reference algorithm, OpenMP) on the same frame."""
+    from oracle import fgs_oracle as orc
+    threads = orc.default_threads()
+    W, H = cam.width, cam.height
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    totals, per_stage, counts, walked = [], None, None, 0
+    for _ in range(max(1, reps)):
+        t0 = time.perf_counter()
+        pre = orc.preprocess(sc.position, sc.shs, sc.opacity, sc.cov3d, W, H, 16, 16, cam.position, cam.rotation,
+                             cam.focal_x, cam.focal_y, cam.zFar, cam.zNear, capacity, threads=threads)
+        t1 = time.perf_counter()
+        K = pre["num_rendered"]
+        ks, vs = orc.sort(K, W, H, 16, 16, pre["keys"], pre["values"], threads=threads)
+        t2 = time.perf_counter()
+        rg = orc.ranges(K, ks, gx * gy)
+        t3 = time.perf_counter()
+        _, _, walked = orc.render(W, H, 16, 16, pre["points_xy"], pre["rgb_depth"], pre["conic_opacity"], vs, rg,
+                                  [0, 0, 0], want_f32=False, threads=threads)
+        t4 = time.perf_counter()
+        totals.append(t4 - t0)
+        if per_stage is None or (t4 - t0) <= min(totals):
+            per_stage = dict(preprocess=(t1 - t0) * 1e3, sort=(t2 - t1) * 1e3, ranges=(t3 - t2) * 1e3, blend=(t4 - t3) * 1e3)
+        counts = pre["counts"]
+    med = statistics.median(totals)
+    return dict(value=1.0 / med, unit="frames/s", cores=threads, kind="port",
+                sample="%d full frame(s) of the benchmark workload, median" % len(totals),
+                ms_per_frame=med * 1e3, stages_ms=per_stage), counts, walked
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build renders on one GPU only; --gpus %d is not supported "
+              "(frames and tile bands are independent, see DESIGN.md for how the path would shard)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from flashgs_amd import cabi, scenes
+
+    cabi.load()   # no library, no benchmark: there is no fallback path
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+
+    sc = scenes.make(args.config)
+    cams = sc.cameras
+    cam = cams[0]
+    W, H = cam.width, cam.height
+    n = sc.num_vertex
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    capacity = {0: 1 << 20, 1: 1 << 22, 2: 1 << 24, 3: 1 << 28, 4: 1 << 25}.get(args.config, 1 << 24)
+
+    def up(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    position, shs, opacity, cov3d = up(sc.position), up(sc.shs), up(sc.opacity), up(sc.cov3d)
+    points_xy = torch.zeros((n, 2), device=dev)
+    rgb_depth = torch.zeros((n, 4), device=dev)
+    conic_opacity = torch.zeros((n, 4), device=dev)
+    keys_u = torch.zeros(capacity, device=dev, dtype=torch.int64)
+    vals_u = torch.zeros(capacity, device=dev, dtype=torch.int32)
+    keys_s = torch.zeros(capacity, device=dev, dtype=torch.int64)
+    vals_s = torch.zeros(capacity, device=dev, dtype=torch.int32)
+    sort_size = cabi.get_sort_buffer_size(capacity)
+    sort_space = torch.zeros(sort_size, device=dev, dtype=torch.int8)
+    ranges = torch.zeros((gx * gy, 2), device=dev, dtype=torch.int32)
+    curr_offset = torch.zeros(1, device=dev, dtype=torch.int32)
+    offset_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+    out_color = torch.zeros((H, W, 3), device=dev, dtype=torch.uint8)
+    bg = np.zeros(3, np.float32)
+    stream = torch.cuda.current_stream().cuda_stream
+    P = {k: v.data_ptr() for k, v in dict(position=position, shs=shs, opacity=opacity, cov3d=cov3d, points_xy=points_xy,
+                                          rgb_depth=rgb_depth, conic_opacity=conic_opacity, keys_u=keys_u, vals_u=vals_u,
+                                          keys_s=keys_s, vals_s=vals_s, sort_space=sort_space, ranges=ranges,
+                                          curr_offset=curr_offset, out_color=out_color).items()}
+
+    def frame(c, ev=None):
+        if ev: ev[0].record()
+        curr_offset.zero_()
+        cabi.preprocess(n, P["position"], P["shs"], P["opacity"], P["cov3d"], W, H, 16, 16, c.position, c.rotation,
+                        c.focal_x, c.focal_y, c.zFar, c.zNear, P["points_xy"], P["rgb_depth"], P["conic_opacity"],
+                        P["keys_u"], P["vals_u"], P["curr_offset"], capacity, stream)
+        if ev: ev[1].record()
+        offset_host.copy_(curr_offset)          # blocking read of the pair count (example.py:79)
+        K = int(offset_host[0])
+        if K < 0 or K >= capacity:
+            raise RuntimeError("too many pairs: %d (capacity %d)" % (K, capacity))
+        if ev: ev[2].record()
+        cabi.sort_gaussian(K, W, H, 16, 16, P["sort_space"], sort_size, P["keys_u"], P["vals_u"], P["keys_s"], P["vals_s"], stream)
+        if ev: ev[3].record()
+        cabi.tile_ranges(16, 16, K, W, H, P["keys_s"], P["ranges"], stream)
+        if ev: ev[4].record()
+        cabi.blend(16, 16, W, H, P["points_xy"], P["rgb_depth"], P["conic_opacity"], P["vals_s"], P["ranges"], bg,
+                   P["out_color"], None, stream)
+        if ev: ev[5].record()
+        return K
+
+    for i in range(args.warmup):
+        frame(cams[i % len(cams)])
+    torch.cuda.synchronize()
+
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(args.steps)]
+    frame_ms, Ks = [], []
+    torch.cuda.synchronize()
+    t_start = time.perf_counter()
+    for i in range(args.steps):
+        t0 = time.perf_counter()
+        Ks.append(frame(cams[i % len(cams)], events[i]))
+        if len(cams) > 1:            # per-frame latency only matters for the trajectory workload
+            torch.cuda.synchronize()
+            frame_ms.append((time.perf_counter() - t0) * 1e3)
+    torch.cuda.synchronize()
+    t_end = time.perf_counter()
+    ms_per_step = (t_end - t_start) * 1e3 / args.steps
+    fps = 1000.0 / ms_per_step
+
+    names = ["preprocess", "readback", "sort", "ranges", "blend"]
+    stage_ms = {nm: statistics.mean(ev[j].elapsed_time(ev[j + 1]) for ev in events) for j, nm in enumerate(names)}
+    K = Ks[0]
+
+    cpu, counts, walked = (None, None, None)
+    if not args.no_cpu_baseline:
+        cpu, counts, walked = cpu_baseline(sc, cam, capacity, args.cpu_reps)
+
+    tiles = gx * gy
+    passes = (32 + int(tiles).bit_length() + 7) // 8
+    stages = {}
+
+    def hbm(name, nbytes):
+        ms = stage_ms[name]
+        gbs = nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+        stages[name] = dict(ms=round(ms, 4), bound="hbm", algorithmic_bytes=int(nbytes),
+                            achieved_GBs=round(gbs, 1), peak_GBs=HBM_PEAK_GBS, frac=round(gbs / HBM_PEAK_GBS, 4))
+
+    if counts is not None and len(cams) == 1:
+        hbm("preprocess", 16 * n + 24 * counts["n_pass"] + 232 * counts["visible"] + 12 * K)
+    else:
+        stages["preprocess"] = dict(ms=round(stage_ms["preprocess"], 4), bound="hbm")
+    hbm("sort", K * (8 + 24 * passes))
+    hbm("ranges", 8 * K + 16 * tiles)
+    stages["readback"] = dict(ms=round(stage_ms["readback"], 4), bound="host latency (4-byte read + sync)")
+
+    blend_ms = stage_ms["blend"]
+    roofline = dict(kernel="blend_kernel<1,1> (16x16 tile, 4 wave64)", bound="valu", achieved=None,
+                    peak=FP32_PEAK_TFLOPS, unit="TFLOP/s", frac=None, traffic=None, launch_ms=round(blend_ms, 4))
+    if walked is not None and len(cams) == 1:
+        evals = 256 * walked
+        tflops = FLOP_PER_EVAL * evals / (blend_ms * 1e-3) / 1e12
+        roofline.update(achieved=round(tflops, 2), frac=round(tflops / FP32_PEAK_TFLOPS, 4),
+                        evaluations=int(evals), flop_per_evaluation=FLOP_PER_EVAL,
+                        issue_slot_frac=round(SLOTS_PER_EVAL * evals / (blend_ms * 1e-3) / LANE_SLOTS_PER_S, 4),
+                        hbm_bytes=int(8 * tiles + 44 * walked + 3 * W * H))
+    stages["blend"] = dict(ms=round(blend_ms, 4), bound="valu")
+
+    result = {
+        "metric": "frames/s, full forward frame (preprocess + sort + ranges + blend)",
+        "value": round(fps, 2), "unit": "frames/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": sc.name, "gaussians": n, "width": W, "height": H, "tile": "16x16",
+                   "sh_degree": 3, "pairs": int(K), "poses": len(cams)},
+        "target_fps": 400 if args.config == 2 else None,
+        "stages": stages,
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    if counts is not None:
+        result["config"].update(n_pass=counts["n_pass"], visible=counts["visible"], walked=int(walked))
+    if frame_ms:
+        frame_ms.sort()
+        result["frame_ms_p50"] = round(frame_ms[len(frame_ms) // 2], 4)
+        result["frame_ms_p99"] = round(frame_ms[min(len(frame_ms) - 1, int(0.99 * len(frame_ms)))], 4)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -26,6 +26,8 @@ SIGNATURES = {
     "fgs_render_32x16": (C.c_int, _RENDER_ARGS),
     "fgs_render_32x32": (C.c_int, _RENDER_ARGS),
     "fgs_render_f32": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 9 + [C.c_void_p]),
+    "fgs_tile_ranges": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 3),
+    "fgs_blend": (C.c_int, [C.c_int] * 4 + [C.c_void_p] * 9),
     "fgs_camera_matrices": (None, [C.c_void_p] * 2 + [C.c_int] * 2 + [C.c_float] * 4 + [C.c_void_p] * 2),
     "fgs_last_error": (C.c_char_p, []),
     "fgs_abi_version": (C.c_int, []),
@@ -113,3 +115,15 @@ def render_f32(block_x, block_y, num_rendered, width, height, points_xy, rgb_dep
     rc = load().fgs_render_f32(block_x, block_y, num_rendered, width, height, points_xy, rgb_depth, conic_opacity,
                                keys_sorted, values_sorted, ranges, bg.ctypes.data, out_u8, out_f32, stream)
     _check(rc, "fgs_render_f32")
+
+
+def tile_ranges(block_x, block_y, num_rendered, width, height, keys_sorted, ranges, stream=0):
+    _check(load().fgs_tile_ranges(block_x, block_y, num_rendered, width, height, keys_sorted, ranges, stream),
+           "fgs_tile_ranges")
+
+
+def blend(block_x, block_y, width, height, points_xy, rgb_depth, conic_opacity, values_sorted, ranges, bg_color,
+          out_u8, out_f32, stream=0):
+    bg = _host_f32(bg_color, 3)
+    _check(load().fgs_blend(block_x, block_y, width, height, points_xy, rgb_depth, conic_opacity, values_sorted,
+                            ranges, bg.ctypes.data, out_u8, out_f32, stream), "fgs_blend")

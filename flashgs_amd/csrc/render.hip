@@ -160,34 +160,56 @@ __global__ __launch_bounds__(kBlendThreads) void blend_kernel(
     }
 }
 
-int render_impl(int sx, int sy, int num_rendered, int width, int height,
-                const float* points_xy, const float* rgb_depth, const float* conic_opacity,
-                const uint64_t* keys_sorted, const uint32_t* values_sorted,
-                int* ranges, const float bg[3], uint8_t* out_u8, float* out_f32, void* stream, const char* who)
+int check_tile(int block_x, int block_y, int* sx, int* sy, const char* who)
+{
+    if ((block_x == 16 && block_y == 16) || (block_x == 32 && block_y == 16) || (block_x == 32 && block_y == 32)) {
+        *sx = block_x / 16;
+        *sy = block_y / 16;
+        return FGS_OK;
+    }
+    return fail(FGS_E_INVALID, "%s: tile %dx%d unsupported (16x16, 32x16, 32x32)", who, block_x, block_y);
+}
+
+// render.cu:556-563: zero the ranges, then mark where each tile starts and ends
+int ranges_impl(int block_x, int block_y, int num_rendered, int width, int height,
+                const uint64_t* keys_sorted, int* ranges, void* stream, const char* who)
 {
     if (num_rendered < 0) return fail(FGS_E_INVALID, "%s: num_rendered = %d is negative", who, num_rendered);
-    if (width <= 0 || height <= 0) return fail(FGS_E_INVALID, "%s: width/height must be positive", who);
-    if (!ranges || !bg || (!out_u8 && !out_f32)) return fail(FGS_E_INVALID, "%s: null ranges, bg_color or output", who);
-    if (num_rendered > 0 && (!points_xy || !rgb_depth || !conic_opacity || !keys_sorted || !values_sorted))
-        return fail(FGS_E_INVALID, "%s: null buffer", who);
-    if (((uintptr_t)rgb_depth | (uintptr_t)conic_opacity) % 16 != 0 ||
-        ((uintptr_t)points_xy | (uintptr_t)keys_sorted | (uintptr_t)ranges) % 8 != 0)
-        return fail(FGS_E_INVALID, "%s: rgb_depth/conic_opacity must be 16-byte aligned, points_xy/keys/ranges 8-byte aligned", who);
-
-    const int bx = 16 * sx, by = 16 * sy;
-    const int tiles_x = (width + bx - 1) / bx, tiles_y = (height + by - 1) / by;     // render.cu:556
+    if (width <= 0 || height <= 0 || block_x <= 0 || block_y <= 0)
+        return fail(FGS_E_INVALID, "%s: width/height/block must be positive", who);
+    if (!ranges || (num_rendered > 0 && !keys_sorted)) return fail(FGS_E_INVALID, "%s: null buffer", who);
+    if (((uintptr_t)keys_sorted | (uintptr_t)ranges) % 8 != 0)
+        return fail(FGS_E_INVALID, "%s: keys and ranges must be 8-byte aligned", who);
+    const int tiles_x = (width + block_x - 1) / block_x, tiles_y = (height + block_y - 1) / block_y;
     const size_t num_tiles = (size_t)tiles_x * tiles_y;
     hipStream_t st = (hipStream_t)stream;
-
-    // render.cu:557
     const size_t words = num_tiles * 2;
     size_t fill_blocks = (words + 1023) / 1024;
     if (fill_blocks > 1024) fill_blocks = 1024;
     hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)fill_blocks), dim3(256), 0, st, ranges, words, 0);
     if (num_rendered > 0)
         hipLaunchKernelGGL(tile_ranges_kernel, dim3((num_rendered + 255) / 256), dim3(256), 0, st,
-                           num_rendered, keys_sorted, (int2*)ranges, (uint32_t)(num_tiles > 0xffffffffu ? 0xffffffffu : num_tiles));
+                           num_rendered, keys_sorted, (int2*)ranges,
+                           (uint32_t)(num_tiles > 0xffffffffu ? 0xffffffffu : num_tiles));
+    return check_hip(hipGetLastError(), who);
+}
 
+// render.cu:566-575
+int blend_impl(int block_x, int block_y, int width, int height,
+               const float* points_xy, const float* rgb_depth, const float* conic_opacity,
+               const uint32_t* values_sorted, const int* ranges, const float bg[3],
+               uint8_t* out_u8, float* out_f32, void* stream, const char* who)
+{
+    int sx = 0, sy = 0;
+    int rc = check_tile(block_x, block_y, &sx, &sy, who);
+    if (rc != FGS_OK) return rc;
+    if (width <= 0 || height <= 0) return fail(FGS_E_INVALID, "%s: width/height must be positive", who);
+    if (!ranges || !bg || (!out_u8 && !out_f32)) return fail(FGS_E_INVALID, "%s: null ranges, bg_color or output", who);
+    if (((uintptr_t)rgb_depth | (uintptr_t)conic_opacity) % 16 != 0 ||
+        ((uintptr_t)points_xy | (uintptr_t)ranges) % 8 != 0)
+        return fail(FGS_E_INVALID, "%s: rgb_depth/conic_opacity must be 16-byte aligned, points_xy/ranges 8-byte aligned", who);
+    const int tiles_x = (width + block_x - 1) / block_x, tiles_y = (height + block_y - 1) / block_y;
+    hipStream_t st = (hipStream_t)stream;
     const dim3 grid(tiles_x, tiles_y);
 #define FGS_LAUNCH_BLEND(SX, SY)                                                                        \
     hipLaunchKernelGGL((blend_kernel<SX, SY>), grid, dim3(kBlendThreads), 0, st,                        \
@@ -196,30 +218,45 @@ int render_impl(int sx, int sy, int num_rendered, int width, int height,
                        bg[0], bg[1], bg[2], out_u8, out_f32)
     if (sx == 1 && sy == 1) FGS_LAUNCH_BLEND(1, 1);
     else if (sx == 2 && sy == 1) FGS_LAUNCH_BLEND(2, 1);
-    else if (sx == 2 && sy == 2) FGS_LAUNCH_BLEND(2, 2);
-    else return fail(FGS_E_INVALID, "%s: tile %dx%d unsupported (16x16, 32x16, 32x32)", who, bx, by);
+    else FGS_LAUNCH_BLEND(2, 2);
 #undef FGS_LAUNCH_BLEND
     return check_hip(hipGetLastError(), who);
+}
+
+int render_impl(int block_x, int block_y, int num_rendered, int width, int height,
+                const float* points_xy, const float* rgb_depth, const float* conic_opacity,
+                const uint64_t* keys_sorted, const uint32_t* values_sorted,
+                int* ranges, const float bg[3], uint8_t* out_u8, float* out_f32, void* stream, const char* who)
+{
+    int sx = 0, sy = 0;
+    int rc = check_tile(block_x, block_y, &sx, &sy, who);
+    if (rc != FGS_OK) return rc;
+    if (num_rendered > 0 && (!points_xy || !rgb_depth || !conic_opacity || !keys_sorted || !values_sorted))
+        return fail(FGS_E_INVALID, "%s: null buffer", who);
+    rc = ranges_impl(block_x, block_y, num_rendered, width, height, keys_sorted, ranges, stream, who);
+    if (rc != FGS_OK) return rc;
+    return blend_impl(block_x, block_y, width, height, points_xy, rgb_depth, conic_opacity, values_sorted, ranges,
+                      bg, out_u8, out_f32, stream, who);
 }
 
 } // namespace
 } // namespace fgs
 
-#define FGS_DEFINE_RENDER(NAME, SX, SY)                                                                      \
+#define FGS_DEFINE_RENDER(NAME, BX, BY)                                                                      \
     extern "C" int NAME(int num_rendered, int width, int height,                                             \
                         const float* points_xy, const float* rgb_depth, const float* conic_opacity,          \
                         const uint64_t* gaussian_keys_sorted, const uint32_t* gaussian_values_sorted,        \
                         int* ranges, const float bg_color[3], uint8_t* out_color, void* stream)              \
     {                                                                                                        \
         if (!out_color) return fgs::fail(FGS_E_INVALID, #NAME ": null out_color");                           \
-        return fgs::render_impl(SX, SY, num_rendered, width, height, points_xy, rgb_depth, conic_opacity,    \
+        return fgs::render_impl(BX, BY, num_rendered, width, height, points_xy, rgb_depth, conic_opacity,    \
                                 gaussian_keys_sorted, gaussian_values_sorted, ranges, bg_color, out_color,   \
                                 nullptr, stream, #NAME);                                                     \
     }
 
-FGS_DEFINE_RENDER(fgs_render_16x16, 1, 1)
-FGS_DEFINE_RENDER(fgs_render_32x16, 2, 1)
-FGS_DEFINE_RENDER(fgs_render_32x32, 2, 2)
+FGS_DEFINE_RENDER(fgs_render_16x16, 16, 16)
+FGS_DEFINE_RENDER(fgs_render_32x16, 32, 16)
+FGS_DEFINE_RENDER(fgs_render_32x32, 32, 32)
 
 extern "C" int fgs_render_f32(int block_x, int block_y, int num_rendered, int width, int height,
                               const float* points_xy, const float* rgb_depth, const float* conic_opacity,
@@ -227,9 +264,23 @@ extern "C" int fgs_render_f32(int block_x, int block_y, int num_rendered, int wi
                               int* ranges, const float bg_color[3], uint8_t* out_color_u8, float* out_color_f32,
                               void* stream)
 {
-    if (block_x % 16 != 0 || block_y % 16 != 0)
-        return fgs::fail(FGS_E_INVALID, "fgs_render_f32: tile %dx%d unsupported (16x16, 32x16, 32x32)", block_x, block_y);
-    return fgs::render_impl(block_x / 16, block_y / 16, num_rendered, width, height, points_xy, rgb_depth,
+    return fgs::render_impl(block_x, block_y, num_rendered, width, height, points_xy, rgb_depth,
                             conic_opacity, gaussian_keys_sorted, gaussian_values_sorted, ranges, bg_color,
                             out_color_u8, out_color_f32, stream, "fgs_render_f32");
+}
+
+extern "C" int fgs_tile_ranges(int block_x, int block_y, int num_rendered, int width, int height,
+                               const uint64_t* gaussian_keys_sorted, int* ranges, void* stream)
+{
+    return fgs::ranges_impl(block_x, block_y, num_rendered, width, height, gaussian_keys_sorted, ranges, stream,
+                            "fgs_tile_ranges");
+}
+
+extern "C" int fgs_blend(int block_x, int block_y, int width, int height,
+                         const float* points_xy, const float* rgb_depth, const float* conic_opacity,
+                         const uint32_t* gaussian_values_sorted, const int* ranges, const float bg_color[3],
+                         uint8_t* out_color_u8, float* out_color_f32, void* stream)
+{
+    return fgs::blend_impl(block_x, block_y, width, height, points_xy, rgb_depth, conic_opacity,
+                           gaussian_values_sorted, ranges, bg_color, out_color_u8, out_color_f32, stream, "fgs_blend");
 }

@@ -1,0 +1,190 @@
+"""Driver with the shape of FlashGS's ``example.py``: ``Scene``, ``Camera``, a statically allocated
+``Rasterizer`` whose ``forward`` runs preprocess -> readback -> sort_gaussian -> render_16x16
+through ``flash_gaussian_splatting.ops``, ``savePpm`` and ``render_scene``.
+
+Differences from the reference driver: the output image is allocated once instead of per frame,
+the too-many-pairs condition raises a real exception (``example.py:82`` raises a string), and the
+tile size is a constructor argument.
+"""
+import json
+import os
+import time
+
+import numpy as np
+import torch
+
+_ops = None
+
+
+def ops():
+    """The compiled operator module; importing it fails loudly if it has not been built."""
+    global _ops
+    if _ops is None:
+        import flash_gaussian_splatting
+        _ops = flash_gaussian_splatting.ops
+    return _ops
+
+
+class Scene:
+    """example.py:10-27"""
+
+    def __init__(self, device):
+        self.device = device
+        self.num_vertex = 0
+        self.position = None
+        self.shs = None
+        self.opacity = None
+        self.cov3d = None
+
+    def loadPly(self, scene_path):
+        self.num_vertex, position, shs, opacity, cov3d = ops().loadPly(scene_path)
+        self._to_device(position, shs, opacity, cov3d)
+
+    def from_arrays(self, position, shs, opacity, cov3d):
+        """Same tensors from host arrays (numpy or torch), e.g. ``flashgs_amd.scenes``."""
+        t = [torch.as_tensor(np.ascontiguousarray(a), dtype=torch.float32) for a in (position, shs, opacity, cov3d)]
+        self.num_vertex = int(t[2].shape[0])
+        self._to_device(*t)
+        return self
+
+    def _to_device(self, position, shs, opacity, cov3d):
+        self.position = position.to(self.device).contiguous()
+        self.shs = shs.to(self.device).contiguous()
+        self.opacity = opacity.to(self.device).contiguous()
+        self.cov3d = cov3d.to(self.device).contiguous()
+
+
+class Camera:
+    """example.py:30-41: one entry of a 3DGS ``cameras.json``."""
+
+    def __init__(self, camera_json):
+        self.id = camera_json.get('id', 0)
+        self.img_name = camera_json.get('img_name', str(self.id))
+        self.width = int(camera_json['width'])
+        self.height = int(camera_json['height'])
+        self.position = torch.tensor(camera_json['position'], dtype=torch.float32)
+        self.rotation = torch.tensor(camera_json['rotation'], dtype=torch.float32)
+        self.focal_x = float(camera_json['fx'])
+        self.focal_y = float(camera_json['fy'])
+        self.zFar = 100.0
+        self.zNear = 0.01
+
+    @classmethod
+    def from_synthetic(cls, cam, cam_id=0):
+        return cls(dict(id=cam_id, img_name="%05d" % cam_id, width=cam.width, height=cam.height,
+                        position=[float(v) for v in cam.position],
+                        rotation=[[float(v) for v in row] for row in np.asarray(cam.rotation).reshape(3, 3)],
+                        fx=cam.focal_x, fy=cam.focal_y))
+
+
+class TooManyPairs(RuntimeError):
+    pass
+
+
+class Rasterizer:
+    """example.py:44-94: all buffers are allocated once, ``forward`` allocates nothing."""
+
+    RENDER = {(16, 16): "render_16x16", (32, 16): "render_32x16", (32, 32): "render_32x32"}
+
+    def __init__(self, scene, MAX_NUM_RENDERED, MAX_NUM_TILES, tile=(16, 16), max_width=0, max_height=0):
+        dev = scene.device
+        self.tile = tuple(tile)
+        self._render = getattr(ops(), self.RENDER[self.tile])
+        self.gaussian_keys_unsorted = torch.zeros(MAX_NUM_RENDERED, device=dev, dtype=torch.int64)
+        self.gaussian_values_unsorted = torch.zeros(MAX_NUM_RENDERED, device=dev, dtype=torch.int32)
+        self.gaussian_keys_sorted = torch.zeros(MAX_NUM_RENDERED, device=dev, dtype=torch.int64)
+        self.gaussian_values_sorted = torch.zeros(MAX_NUM_RENDERED, device=dev, dtype=torch.int32)
+        self.MAX_NUM_RENDERED = MAX_NUM_RENDERED
+        self.MAX_NUM_TILES = MAX_NUM_TILES
+        self.SORT_BUFFER_SIZE = ops().get_sort_buffer_size(MAX_NUM_RENDERED)
+        self.list_sorting_space = torch.zeros(self.SORT_BUFFER_SIZE, device=dev, dtype=torch.int8)
+        self.ranges = torch.zeros((MAX_NUM_TILES, 2), device=dev, dtype=torch.int32)
+        self.curr_offset = torch.zeros(1, device=dev, dtype=torch.int32)
+        self.points_xy = torch.zeros((scene.num_vertex, 2), device=dev, dtype=torch.float32)
+        self.rgb_depth = torch.zeros((scene.num_vertex, 4), device=dev, dtype=torch.float32)
+        self.conic_opacity = torch.zeros((scene.num_vertex, 4), device=dev, dtype=torch.float32)
+        self._offset_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        self._out = None
+        if max_width and max_height:
+            self._out = torch.zeros((max_height, max_width, 3), device=dev, dtype=torch.uint8)
+        self.num_rendered = 0
+
+    def _image(self, camera, device):
+        if self._out is None or self._out.shape[0] != camera.height or self._out.shape[1] != camera.width:
+            self._out = torch.zeros((camera.height, camera.width, 3), device=device, dtype=torch.uint8)
+        return self._out
+
+    def forward(self, scene, camera, bg_color):
+        o = ops()
+        bx, by = self.tile
+        tiles = ((camera.width + bx - 1) // bx) * ((camera.height + by - 1) // by)
+        if tiles > self.MAX_NUM_TILES:
+            raise ValueError("image needs %d tiles, MAX_NUM_TILES is %d" % (tiles, self.MAX_NUM_TILES))
+        self.curr_offset.zero_()
+        o.preprocess(scene.position, scene.shs, scene.opacity, scene.cov3d,
+                     camera.width, camera.height, bx, by,
+                     camera.position, camera.rotation,
+                     camera.focal_x, camera.focal_y, camera.zFar, camera.zNear,
+                     self.points_xy, self.rgb_depth, self.conic_opacity,
+                     self.gaussian_keys_unsorted, self.gaussian_values_unsorted, self.curr_offset)
+        # the one blocking device-to-host read of the frame (example.py:79)
+        self._offset_host.copy_(self.curr_offset, non_blocking=False)
+        num_rendered = int(self._offset_host[0])
+        self.num_rendered = num_rendered
+        if num_rendered < 0 or num_rendered >= self.MAX_NUM_RENDERED:
+            raise TooManyPairs("Too many k-v pairs! (%d, capacity %d)" % (num_rendered, self.MAX_NUM_RENDERED))
+        o.sort_gaussian(num_rendered, camera.width, camera.height, bx, by, self.list_sorting_space,
+                        self.gaussian_keys_unsorted, self.gaussian_values_unsorted,
+                        self.gaussian_keys_sorted, self.gaussian_values_sorted)
+        out_color = self._image(camera, scene.device)
+        self._render(num_rendered, camera.width, camera.height,
+                     self.points_xy, self.rgb_depth, self.conic_opacity,
+                     self.gaussian_keys_sorted, self.gaussian_values_sorted,
+                     self.ranges, bg_color, out_color)
+        return out_color
+
+
+def savePpm(image, path):
+    """example.py:97-102: binary P6."""
+    image = image.cpu()
+    assert image.dim() >= 3 and image.size(2) == 3
+    with open(path, 'wb') as f:
+        f.write(b'P6\n' + f'{image.size(1)} {image.size(0)}\n255\n'.encode() + image.numpy().tobytes())
+
+
+def render_scene(model_path, test_performance=False, device='cuda:0', MAX_NUM_RENDERED=2 ** 27, MAX_NUM_TILES=2 ** 20):
+    """example.py:105-144: render every camera of ``<model_path>/cameras.json`` to ``test_out/*.ppm``."""
+    scene_path = os.path.join(model_path, "point_cloud", "iteration_30000", "point_cloud.ply")
+    camera_path = os.path.join(model_path, "cameras.json")
+    device = torch.device(device)
+    bg_color = torch.zeros(3, dtype=torch.float32)
+    scene = Scene(device)
+    scene.loadPly(scene_path)
+    print("num_vertex = %d" % scene.num_vertex)
+    with open(camera_path, 'r') as camera_file:
+        cameras_json = json.load(camera_file)
+    image_dir = os.path.join(model_path, "test_out")
+    os.makedirs(image_dir, exist_ok=True)
+    rasterizer = Rasterizer(scene, MAX_NUM_RENDERED, MAX_NUM_TILES)
+    for camera_json in cameras_json:
+        camera = Camera(camera_json)
+        print("image name = %s" % camera.img_name)
+        image = rasterizer.forward(scene, camera, bg_color)
+        if test_performance:
+            n = 10
+            torch.cuda.synchronize()
+            t0 = time.time()
+            for _ in range(n):
+                image = rasterizer.forward(scene, camera, bg_color)
+            torch.cuda.synchronize()
+            t1 = time.time()
+            print("elapsed time = %f ms" % ((t1 - t0) / n * 1000))
+            print("fps = %f" % (n / (t1 - t0)))
+        savePpm(image, os.path.join(image_dir, "%s.ppm" % camera.img_name))
+
+
+if __name__ == "__main__":
+    import sys
+    if len(sys.argv) < 2:
+        sys.exit("usage: python -m flashgs_amd.rasterizer <model_path>")
+    render_scene(sys.argv[1], True)

@@ -106,6 +106,19 @@ int fgs_render_f32(int block_x, int block_y, int num_rendered, int width, int he
                    void* stream);
 
 /*
+ * The two halves of fgs_render_*, for callers that want them separately (per-stage timing, or
+ * blending several images from one set of ranges).  fgs_tile_ranges is render.cu:556-563 (zero
+ * `ranges`, then identifyTileRanges, render.cu:9-31); fgs_blend is the renderCUDA launch of
+ * render.cu:566-575 reading `ranges`.  Either output of fgs_blend may be NULL, not both.
+ */
+int fgs_tile_ranges(int block_x, int block_y, int num_rendered, int width, int height,
+                    const uint64_t* gaussian_keys_sorted, int* ranges, void* stream);
+int fgs_blend(int block_x, int block_y, int width, int height,
+              const float* points_xy, const float* rgb_depth, const float* conic_opacity,
+              const uint32_t* gaussian_values_sorted, const int* ranges, const float bg_color[3],
+              uint8_t* out_color_u8, float* out_color_f32, void* stream);
+
+/*
  * Host-side camera set-up used by fgs_preprocess (preprocess.cu:420-448,461-466), exposed so
  * callers and tests can inspect it: column-major 4x4 view and projection matrices.
  */
