@@ -8,7 +8,7 @@
  *
  * Pin status (what checks each function independently of this file; the tests
  * named live in tests/test_oracle_*.py):
- *   log2f                 float64 numpy log2, <= 2 ulp over 1e6 samples        pinned
+ *   log2f                 float64 numpy log2, <= 4 ulp over 25k samples         pinned
  *   view_proj             closed forms (identity rotation, fx/W), float64      pinned
  *   cov2d                 float64 EWA model J W S W^T J^T + 0.3 I, closed form pinned
  *   conic/power/radius    closed forms ln(256 op), floor(sqrt(2 p c)+1)        pinned
