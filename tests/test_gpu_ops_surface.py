@@ -1,0 +1,87 @@
+"""The op surface on the GPU, used the way FlashGS's example.py uses it: ``Rasterizer.forward``
+through ``flash_gaussian_splatting.ops`` against the oracle, and the error behaviour of the ops."""
+import numpy as np
+import pytest
+import torch
+
+from flashgs_amd import scenes
+from flashgs_amd.rasterizer import Camera, Rasterizer, Scene, TooManyPairs, savePpm
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup(n=40_000, cap=1 << 19, tile=(16, 16)):
+    sc = scenes.config0(n=n)
+    scene = Scene(torch.device("cuda:0")).from_arrays(sc.position, sc.shs, sc.opacity, sc.cov3d)
+    return sc, scene, Camera.from_synthetic(sc.cameras[0]), Rasterizer(scene, cap, 1 << 14, tile=tile)
+
+
+@pytest.mark.parametrize("tile", [(16, 16), (32, 16), (32, 32)])
+def test_rasterizer_forward_matches_oracle(oracle, tile, tmp_path):
+    sc, scene, cam, rast = _setup(tile=tile)
+    c0 = sc.cameras[0]
+    bg = torch.tensor([0.0, 0.2, 0.4])
+    img = rast.forward(scene, cam, bg)
+    img2 = rast.forward(scene, cam, bg).cpu().numpy()          # a second frame reuses every buffer
+    K = rast.num_rendered
+    pre = oracle.preprocess(sc.position, sc.shs, sc.opacity, sc.cov3d, c0.width, c0.height, tile[0], tile[1],
+                            c0.position, c0.rotation, c0.focal_x, c0.focal_y, c0.zFar, c0.zNear, 1 << 19)
+    assert pre["num_rendered"] == K
+    ks, vs = oracle.sort(K, c0.width, c0.height, tile[0], tile[1], pre["keys"], pre["values"])
+    assert np.array_equal(rast.gaussian_keys_sorted[:K].cpu().numpy().view(np.uint64), ks)
+    assert np.array_equal(rast.gaussian_values_sorted[:K].cpu().numpy().view(np.uint32), vs)
+    gx, gy = (c0.width + tile[0] - 1) // tile[0], (c0.height + tile[1] - 1) // tile[1]
+    rg = oracle.ranges(K, ks, gx * gy)
+    assert np.array_equal(rast.ranges[:gx * gy].cpu().numpy(), rg)
+    u8, _, _ = oracle.render(c0.width, c0.height, tile[0], tile[1], pre["points_xy"], pre["rgb_depth"],
+                             pre["conic_opacity"], vs, rg, bg.numpy(), want_f32=False)
+    d = np.abs(img2.astype(np.int16) - u8.astype(np.int16))
+    assert d.max() <= 1 and (d > 0).mean() < 0.01
+    path = tmp_path / "frame.ppm"
+    savePpm(img, str(path))
+    data = path.read_bytes()
+    assert data.startswith(b"P6\n%d %d\n255\n" % (c0.width, c0.height))
+
+
+def test_int8_image_like_the_reference_driver():
+    """example.py:89 allocates the image as int8; the op accepts any 1-byte dtype."""
+    import flash_gaussian_splatting as fgs
+    sc, scene, cam, rast = _setup(n=5000)
+    bg = torch.zeros(3)
+    ref = rast.forward(scene, cam, bg).clone()
+    out = torch.zeros((cam.height, cam.width, 3), device="cuda:0", dtype=torch.int8)
+    fgs.ops.render_16x16(rast.num_rendered, cam.width, cam.height, rast.points_xy, rast.rgb_depth, rast.conic_opacity,
+                         rast.gaussian_keys_sorted, rast.gaussian_values_sorted, rast.ranges, bg, out)
+    assert torch.equal(out.view(torch.uint8), ref)
+
+
+def test_too_many_pairs_raises():
+    sc, scene, cam, _ = _setup(n=40_000)
+    small = Rasterizer(scene, 1000, 1 << 14)
+    with pytest.raises(TooManyPairs):
+        small.forward(scene, cam, torch.zeros(3))
+
+
+def test_ops_errors_on_the_gpu():
+    import flash_gaussian_splatting as fgs
+    sc, scene, cam, rast = _setup(n=5000)
+    rast.forward(scene, cam, torch.zeros(3))
+    K = rast.num_rendered
+    tiny = torch.zeros(64, device="cuda:0", dtype=torch.int8)
+    with pytest.raises(RuntimeError, match="needed"):            # workspace too small
+        fgs.ops.sort_gaussian(K, cam.width, cam.height, 16, 16, tiny, rast.gaussian_keys_unsorted,
+                              rast.gaussian_values_unsorted, rast.gaussian_keys_sorted, rast.gaussian_values_sorted)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        fgs.ops.preprocess(scene.position, scene.shs, scene.opacity, scene.cov3d, cam.width, cam.height, 16, 16,
+                           cam.position, cam.rotation, cam.focal_x, cam.focal_y, cam.zFar, cam.zNear,
+                           torch.zeros((scene.num_vertex, 4), device="cuda:0")[:, :2], rast.rgb_depth, rast.conic_opacity,
+                           rast.gaussian_keys_unsorted, rast.gaussian_values_unsorted, rast.curr_offset)
+    with pytest.raises(RuntimeError, match="dtype"):
+        fgs.ops.preprocess(scene.position, scene.shs, scene.opacity, scene.cov3d, cam.width, cam.height, 16, 16,
+                           cam.position, cam.rotation, cam.focal_x, cam.focal_y, cam.zFar, cam.zNear,
+                           rast.points_xy, rast.rgb_depth, rast.conic_opacity,
+                           rast.gaussian_keys_unsorted.to(torch.int32), rast.gaussian_values_unsorted, rast.curr_offset)
+    with pytest.raises(RuntimeError, match="too small"):
+        fgs.ops.render_16x16(K, cam.width, cam.height, rast.points_xy, rast.rgb_depth, rast.conic_opacity,
+                             rast.gaussian_keys_sorted, rast.gaussian_values_sorted, rast.ranges[:10], torch.zeros(3),
+                             torch.zeros((cam.height, cam.width, 3), device="cuda:0", dtype=torch.uint8))

@@ -71,3 +71,168 @@ def test_config0_full_frame(oracle):
 def test_small_scene_white_background(oracle):
     sc = scenes.config0(n=5000)
     _check_frame(oracle, sc, sc.cameras[0], 1 << 16, bg=(1.0, 0.5, 0.25))
+
+
+def test_config1_partial_tile_rows(oracle):
+    """1920x1080: the last tile row is half outside the image."""
+    sc = scenes.make(1, n=200_000)
+    _check_frame(oracle, sc, sc.cameras[0], 1 << 20)
+
+
+def _big_splat_scene(n=4000, seed=7):
+    """Splats whose candidate rectangles exceed 64 tiles, so the whole-wave tile test runs."""
+    sc = scenes.config0(n=n)
+    rng = np.random.default_rng(seed)
+    ls = rng.normal(-2.2, 0.9, (n, 3))
+    ls[: n // 50] += 2.5                      # a few enormous ones, some covering the screen
+    sc.cov3d = scenes.cov3d_from_scale_rotation(np.exp(ls).astype(np.float32), scenes._unit_quats(rng, n))
+    return sc
+
+
+@pytest.mark.parametrize("block", [(16, 16), (32, 16), (32, 32)])
+def test_large_splats_all_tile_sizes(oracle, block):
+    sc = _big_splat_scene()
+    cam = sc.cameras[0]
+    cam.width, cam.height = 1000, 600            # neither a multiple of 16 nor of 32
+    ref = _check_frame(oracle, sc, cam, 1 << 22, block=block, bg=(0.3, 0.1, 0.9))
+    assert ref["pre"]["counts"]["candidates"] > 64 * 20
+
+
+def test_anisotropic_splats_near_camera(oracle):
+    """Needle-shaped splats close to the camera: the exact ellipse test rejects most candidates."""
+    sc = scenes.config4(n=60_000, width=1280, height=720, n_poses=3)
+    for cam in sc.cameras:
+        ref = _check_frame(oracle, sc, cam, 1 << 22)
+        assert ref["K"] < ref["pre"]["counts"]["candidates"]
+
+
+def test_empty_inputs(oracle):
+    import gpu_pipeline as gp
+    import torch
+    from flashgs_amd import cabi
+    # no Gaussian survives the culls: zero pairs, background image, ranges all zero
+    sc = scenes.config0(n=1000)
+    sc.position[:, 2] = -100.0                    # all behind the camera
+    ref = _check_frame(oracle, sc, sc.cameras[0], 1 << 10, bg=(0.25, 0.5, 0.75))
+    assert ref["K"] == 0
+    # P == 0 is accepted and leaves the counter alone
+    off = torch.full((1,), 5, device=gp.DEV, dtype=torch.int32)
+    cabi.preprocess(0, 0, 0, 0, 0, 64, 64, 16, 16, [0, 0, 0], np.eye(3), 50.0, 50.0, 100.0, 0.01, 0, 0, 0, 0, 0,
+                    off.data_ptr(), 16, 0)
+    assert int(off.cpu()[0]) == 5
+
+
+def test_start_offset_and_capacity_guard(oracle):
+    """Pairs are appended after the caller's starting offset (preprocess.cu:330,395 add to the
+    counter); pairs beyond key_capacity are dropped but still counted."""
+    import gpu_pipeline as gp
+    sc = scenes.config0(n=30_000)
+    cam = sc.cameras[0]
+    sd = gp.SceneOnDevice(sc)
+    full = gp.preprocess(sd, cam, 1 << 18)
+    K = full["num_rendered"]
+    assert K > 1000
+    shifted = gp.preprocess(sd, cam, 1 << 18, start_offset=777)
+    assert shifted["num_rendered"] == K + 777
+    assert np.array_equal(gp.u64(shifted["keys"])[777:777 + K], gp.u64(full["keys"])[:K])
+    assert np.all(gp.u64(shifted["keys"])[:777] == 0)
+    cap = K // 2
+    n = sd.n
+    import torch
+    keys = torch.zeros(cap + 64, device=gp.DEV, dtype=torch.int64)
+    values = torch.full((cap + 64,), -1, device=gp.DEV, dtype=torch.int32)
+    off = torch.zeros(1, device=gp.DEV, dtype=torch.int32)
+    from flashgs_amd import cabi
+    cabi.preprocess(n, sd.position.data_ptr(), sd.shs.data_ptr(), sd.opacity.data_ptr(), sd.cov3d.data_ptr(),
+                    cam.width, cam.height, 16, 16, cam.position, cam.rotation, cam.focal_x, cam.focal_y, cam.zFar, cam.zNear,
+                    full["points_xy"].data_ptr(), full["rgb_depth"].data_ptr(), full["conic_opacity"].data_ptr(),
+                    keys.data_ptr(), values.data_ptr(), off.data_ptr(), cap, 0)
+    torch.cuda.synchronize()
+    assert int(off.cpu()[0]) == K                                     # still the full count
+    assert np.array_equal(gp.u64(keys)[:cap], gp.u64(full["keys"])[:cap])
+    assert np.all(gp.u64(keys)[cap:] == 0) and np.all(values.cpu().numpy()[cap:] == -1)   # nothing past the capacity
+
+
+def test_repeated_frames_are_deterministic():
+    import gpu_pipeline as gp
+    sc = scenes.config0(n=50_000)
+    cam = sc.cameras[0]
+    sd = gp.SceneOnDevice(sc)
+    first = gp.preprocess(sd, cam, 1 << 18)
+    K = first["num_rendered"]
+    ks0, vs0 = gp.sort(K, cam.width, cam.height, first["keys"], first["values"])
+    for _ in range(5):
+        again = gp.preprocess(sd, cam, 1 << 18)
+        assert again["num_rendered"] == K
+        assert np.array_equal(gp.u64(again["keys"])[:K], gp.u64(first["keys"])[:K])
+        ks, vs = gp.sort(K, cam.width, cam.height, again["keys"], again["values"], space_for=1 << 18)
+        assert np.array_equal(gp.u64(ks)[:K], gp.u64(ks0)[:K]) and np.array_equal(gp.u32(vs)[:K], gp.u32(vs0)[:K])
+
+
+@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 2047, 2048, 2049, 4096, 100_003, 1_500_000])
+def test_sort_sizes_against_numpy(n):
+    """Ragged sizes around the wave (64) and workgroup tile (2048) boundaries, with many equal keys."""
+    import gpu_pipeline as gp
+    rng = np.random.default_rng(n)
+    W, H = 3840, 2160
+    tiles = 240 * 135
+    tile = rng.integers(0, tiles, n).astype(np.uint64)
+    depth = rng.uniform(0.2, 80.0, n).astype(np.float32)
+    if n > 100:
+        depth[: n // 3] = depth[0]
+        tile[: n // 5] = tile[1]
+    keys = (tile << np.uint64(32)) | depth.view(np.uint32).astype(np.uint64)
+    vals = rng.permutation(n).astype(np.uint32)
+    ks, vs = gp.sort(n, W, H, gp.dev(keys.view(np.int64)), gp.dev(vals.view(np.int32)))
+    order = np.argsort(keys, kind="stable")
+    assert np.array_equal(gp.u64(ks)[:n], keys[order])
+    assert np.array_equal(gp.u32(vs)[:n], vals[order])
+
+
+def test_sort_full_size_properties():
+    """At the headline size (8M pairs, 47 key bits) without the oracle: output is a permutation of
+    the input, non-decreasing, and equal keys keep their input order."""
+    import gpu_pipeline as gp
+    import torch
+    n = 8_115_406
+    g = torch.Generator(device=gp.DEV).manual_seed(1)
+    tile = torch.randint(0, 32400, (n,), device=gp.DEV, generator=g, dtype=torch.int64)
+    depth = (torch.rand(n, device=gp.DEV, generator=g) * 60 + 0.2).to(torch.float32).view(torch.int32).to(torch.int64)
+    depth[: n // 4] = depth[0]
+    keys = (tile << 32) | depth
+    vals = torch.arange(n, device=gp.DEV, dtype=torch.int32)        # value = input position
+    ks, vs = gp.sort(n, 3840, 2160, keys, vals)
+    assert bool((ks[1:] >= ks[:-1]).all())
+    assert bool((keys[vs.long()] == ks).all())                        # pairs stayed together
+    tie = ks[1:] == ks[:-1]
+    assert bool((vs[1:][tie] > vs[:-1][tie]).all())                   # stable
+    assert int(torch.bincount(vs.long(), minlength=n).max()) == 1     # a permutation
+
+
+def test_ranges_kernel_against_searchsorted():
+    import gpu_pipeline as gp
+    import torch
+    from flashgs_amd import cabi
+    rng = np.random.default_rng(33)
+    W, H = 1920, 1080
+    tiles = 120 * 68
+    for n in (0, 1, 5, 70_001):
+        tile = np.sort(rng.integers(0, tiles, n)).astype(np.uint64)
+        tile = tile[(tile < 1000) | (tile > 1300)]
+        n = tile.size
+        keys = (tile << np.uint64(32)) | rng.integers(0, 1 << 32, n).astype(np.uint64)
+        dk = gp.dev(keys.view(np.int64)) if n else torch.zeros(1, device=gp.DEV, dtype=torch.int64)
+        rg = torch.full((tiles, 2), -9, device=gp.DEV, dtype=torch.int32)
+        cabi.tile_ranges(16, 16, n, W, H, dk.data_ptr(), rg.data_ptr(), 0)
+        torch.cuda.synchronize()
+        lo = np.searchsorted(tile, np.arange(tiles), side="left")
+        hi = np.searchsorted(tile, np.arange(tiles), side="right")
+        want = np.where((lo == hi)[:, None], 0, np.stack([lo, hi], 1)).astype(np.int32)
+        assert np.array_equal(rg.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("config", [1, 2])
+def test_full_size_configs(oracle, config):
+    """The 1080p / 1M and the 4K / 3M configurations end to end against the oracle."""
+    sc = scenes.make(config)
+    _check_frame(oracle, sc, sc.cameras[0], 1 << 24)
