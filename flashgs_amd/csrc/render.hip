@@ -3,21 +3,19 @@
 // Replaces FlashGS render<BX,BY> (csrc/cuda_rasterizer/render.cu:549-576): zero the ranges,
 // identifyTileRanges (:9-31) and renderCUDA (:199-547).
 //
-// Blend layout: a workgroup of 256 threads (4 wave64) owns one tile.  A tile is made of
-// 16x16-pixel sub-tiles (1 for 16x16, 2 for 32x16, 4 for 32x32); each wave owns the same 8x8
-// quadrant of every sub-tile, so a thread shades one pixel per sub-tile.  Gaussians are staged
-// 256 at a time into LDS by all threads together (index -> centre, conic+opacity, colour), then
-// every wave walks the batch reading LDS at a wave-uniform address.  After every second Gaussian
-// (the reference tests after each pair, render.cu:394-405) a wave checks with one ballot whether
-// all of its pixels have T < 1e-4 and stops shading if so; the workgroup leaves when all four
-// waves have stopped or the range is exhausted.
+// Blend layout: one wave64 owns one tile.  A tile is made of 16x16-pixel sub-tiles (1 for 16x16,
+// 2 for 32x16, 4 for 32x32); lane l shades the 2x2 pixel quad at (2*(l%8), 2*(l/8)) of every
+// sub-tile, so the quadratic form is evaluated with shared column/row terms.  Gaussians are
+// staged 64 at a time into LDS (one per lane: index -> centre, conic+opacity, colour) while the
+// loads of the following batch are already in flight, and the wave walks the batch reading LDS
+// at wave-uniform addresses.  After every second Gaussian one ballot tests whether all pixels of
+// the tile have T < 1e-4, which is the reference's stop rule (render.cu:394-408).  A workgroup is
+// a single wave, so no workgroup barrier is needed anywhere.
 #include "fgs_internal.h"
 
 namespace fgs {
 namespace {
 
-constexpr int kBlendThreads = 256;
-constexpr int kBatch = 256;
 
 __global__ __launch_bounds__(256) void fill_i32_kernel(int* p, size_t n, int v)
 {
@@ -55,8 +53,41 @@ __device__ __forceinline__ uint8_t encode_u8(float x)
     return (uint8_t)v;
 }
 
+// One Gaussian applied to this lane's 2x2 pixel quad (render.cu:40-52 for each pixel).  The
+// quadratic is split into a column part A[i], a row part B[j] and the cross term, so the four
+// evaluations share most of the arithmetic.
+struct Quad {
+    float T[2][2], r[2][2], g[2][2], b[2][2];
+};
+
+__device__ __forceinline__ void shade_quad(Quad& q, float px0, float py0, const float4 a, const float4 b4, const float blue)
+{
+    // a = (centre x, centre y, conic x, conic y), b4 = (conic z, log2 opacity, red, green)
+    const float dx0 = a.x - px0, dx1 = a.x - (px0 + 1.0f);
+    const float dy0 = a.y - py0, dy1 = a.y - (py0 + 1.0f);
+    const float A0 = a.z * dx0 * dx0, A1 = a.z * dx1 * dx1;
+    const float B0 = b4.y + b4.x * dy0 * dy0, B1 = b4.y + b4.x * dy1 * dy1;
+    const float E0 = a.w * dx0, E1 = a.w * dx1;
+    float pw[2][2];
+    pw[0][0] = (A0 + B0) + E0 * dy0;
+    pw[0][1] = (A1 + B0) + E1 * dy0;
+    pw[1][0] = (A0 + B1) + E0 * dy1;
+    pw[1][1] = (A1 + B1) + E1 * dy1;
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const float alpha = __builtin_amdgcn_exp2f(pw[j][i]);
+            const float at = alpha * q.T[j][i];
+            q.r[j][i] += b4.z * at;
+            q.g[j][i] += b4.w * at;
+            q.b[j][i] += blue * at;
+            q.T[j][i] -= at;
+        }
+}
+
 template <int SX, int SY>
-__global__ __launch_bounds__(kBlendThreads) void blend_kernel(
+__global__ __launch_bounds__(kWave) void blend_kernel(
     const int2* __restrict__ ranges,
     const uint32_t* __restrict__ point_list,
     int width, int height, int tiles_x,
@@ -67,97 +98,104 @@ __global__ __launch_bounds__(kBlendThreads) void blend_kernel(
     uint8_t* __restrict__ out_u8,
     float* __restrict__ out_f32)
 {
-    constexpr int kSub = SX * SY;              // pixels per thread
-    __shared__ float2 s_xy[kBatch];
-    __shared__ float4 s_co[kBatch];
-    __shared__ float4 s_rgb[kBatch];
-    __shared__ int s_waves_done;
+    constexpr int kSub = SX * SY;              // 16x16 sub-tiles per tile = quads per lane
+    __shared__ float4 s_a[kWave];              // centre x, centre y, conic x, conic y
+    __shared__ float4 s_b[kWave];              // conic z, log2 opacity, red, green
+    __shared__ float s_c[kWave];               // blue
 
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
-    const int wave = tid / kWave;
+    const int lane = threadIdx.x;
     const int tile_x = blockIdx.x, tile_y = blockIdx.y;
     const int2 range = ranges[tile_y * tiles_x + tile_x];
-
-    // this thread's pixel inside a 16x16 sub-tile: wave -> 8x8 quadrant, lane -> pixel of it
-    const int lx = (wave & 1) * 8 + (lane & 7);
-    const int ly = (wave >> 1) * 8 + (lane >> 3);
-    int pix_x[kSub], pix_y[kSub];
-    float pxf[kSub], pyf[kSub];
-#pragma unroll
-    for (int s = 0; s < kSub; s++) {
-        pix_x[s] = tile_x * (16 * SX) + (s % SX) * 16 + lx;
-        pix_y[s] = tile_y * (16 * SY) + (s / SX) * 16 + ly;
-        pxf[s] = (float)pix_x[s];
-        pyf[s] = (float)pix_y[s];
-    }
-
-    float T[kSub], Cr[kSub], Cg[kSub], Cb[kSub];
-#pragma unroll
-    for (int s = 0; s < kSub; s++) { T[s] = 1.0f; Cr[s] = 0.0f; Cg[s] = 0.0f; Cb[s] = 0.0f; }
-
-    if (tid == 0) s_waves_done = 0;
-    bool wave_done = false;
     const int n = range.y - range.x;
 
-    for (int base = 0; base < n; base += kBatch) {
-        const int cnt = min(kBatch, n - base);
-        __syncthreads();                       // previous batch fully consumed; s_waves_done initialised
-        if (s_waves_done == kBlendThreads / kWave) break;
-        if (tid < cnt) {
-            const uint32_t g = point_list[range.x + base + tid];
-            s_xy[tid] = points_xy[g];
-            s_co[tid] = conic_opacity[g];
-            s_rgb[tid] = rgb_depth[g];
-        }
-        __syncthreads();
-        if (!wave_done) {
-            for (int j = 0; j < cnt; j++) {
-                const float2 g = s_xy[j];
-                const float4 co = s_co[j];
-                const float4 col = s_rgb[j];
+    // lane -> 2x2 quad of every 16x16 sub-tile
+    const int qx = (lane & 7) * 2, qy = (lane >> 3) * 2;
+    int pix_x[kSub], pix_y[kSub];
+    float pxf[kSub], pyf[kSub];
+    Quad quad[kSub];
 #pragma unroll
-                for (int s = 0; s < kSub; s++) {       // render.cu:40-52
-                    const float dx = g.x - pxf[s], dy = g.y - pyf[s];
-                    const float power = co.w + co.x * dx * dx + co.z * dy * dy + co.y * dx * dy;
-                    const float alpha = __builtin_amdgcn_exp2f(power);
-                    const float at = alpha * T[s];
-                    Cr[s] += col.x * at;
-                    Cg[s] += col.y * at;
-                    Cb[s] += col.z * at;
-                    T[s] -= at;
-                }
-                if (j & 1) {
-                    bool done = true;
+    for (int s = 0; s < kSub; s++) {
+        pix_x[s] = tile_x * (16 * SX) + (s % SX) * 16 + qx;
+        pix_y[s] = tile_y * (16 * SY) + (s / SX) * 16 + qy;
+        pxf[s] = (float)pix_x[s];
+        pyf[s] = (float)pix_y[s];
 #pragma unroll
-                    for (int s = 0; s < kSub; s++) done = done && T[s] < 0.0001f;
-                    if (ballot(!done) == 0) { wave_done = true; break; }
-                }
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                quad[s].T[j][i] = 1.0f;
+                quad[s].r[j][i] = 0.0f; quad[s].g[j][i] = 0.0f; quad[s].b[j][i] = 0.0f;
             }
-            if (wave_done && lane == 0) atomicAdd(&s_waves_done, 1);
+    }
+
+    // registers hold the batch that is staged next; loads for it overlap the shading of the current one
+    float2 nxy = make_float2(0.f, 0.f);
+    float4 nco = make_float4(0.f, 0.f, 0.f, 0.f), nrgb = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (lane < n) {
+        const uint32_t g = point_list[range.x + lane];
+        nxy = points_xy[g]; nco = conic_opacity[g]; nrgb = rgb_depth[g];
+    }
+
+    bool done = false;
+    for (int base = 0; base < n && !done; base += kWave) {
+        const int cnt = min(kWave, n - base);
+        __builtin_amdgcn_wave_barrier();
+        s_a[lane] = make_float4(nxy.x, nxy.y, nco.x, nco.y);
+        s_b[lane] = make_float4(nco.z, nco.w, nrgb.x, nrgb.y);
+        s_c[lane] = nrgb.z;
+        __builtin_amdgcn_wave_barrier();
+        if (base + kWave + lane < n) {
+            const uint32_t g = point_list[range.x + base + kWave + lane];
+            nxy = points_xy[g]; nco = conic_opacity[g]; nrgb = rgb_depth[g];
+        }
+        // Gaussians go in pairs; the tile-wide stop is tested after each pair (render.cu:394-408)
+        for (int j = 0; j < cnt; j += 2) {
+            {
+                const float4 a = s_a[j], b4 = s_b[j];
+                const float blue = s_c[j];
+#pragma unroll
+                for (int s = 0; s < kSub; s++) shade_quad(quad[s], pxf[s], pyf[s], a, b4, blue);
+            }
+            if (j + 1 >= cnt) break;            // odd tail (render.cu:486-487)
+            {
+                const float4 a = s_a[j + 1], b4 = s_b[j + 1];
+                const float blue = s_c[j + 1];
+#pragma unroll
+                for (int s = 0; s < kSub; s++) shade_quad(quad[s], pxf[s], pyf[s], a, b4, blue);
+            }
+            float tmax = 0.0f;
+#pragma unroll
+            for (int s = 0; s < kSub; s++)
+                tmax = fmaxf(tmax, fmaxf(fmaxf(quad[s].T[0][0], quad[s].T[0][1]), fmaxf(quad[s].T[1][0], quad[s].T[1][1])));
+            if (ballot(!(tmax < 0.0001f)) == 0) { done = true; break; }
         }
     }
 
     // render.cu:59-73
 #pragma unroll
-    for (int s = 0; s < kSub; s++) {
-        if (pix_x[s] < width && pix_y[s] < height) {
-            const size_t pid = (size_t)width * pix_y[s] + pix_x[s];
-            float t = T[s];
-            if (t < 0.0001f) t = 0.0f;
-            const float r = Cr[s] + t * bg_r, g = Cg[s] + t * bg_g, b = Cb[s] + t * bg_b;
-            if (out_u8) {
-                out_u8[3 * pid + 0] = encode_u8(r);
-                out_u8[3 * pid + 1] = encode_u8(g);
-                out_u8[3 * pid + 2] = encode_u8(b);
+    for (int s = 0; s < kSub; s++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const int x = pix_x[s] + i, y = pix_y[s] + j;
+                if (x < width && y < height) {
+                    const size_t pid = (size_t)width * y + x;
+                    float t = quad[s].T[j][i];
+                    if (t < 0.0001f) t = 0.0f;
+                    const float r = quad[s].r[j][i] + t * bg_r, g = quad[s].g[j][i] + t * bg_g, b = quad[s].b[j][i] + t * bg_b;
+                    if (out_u8) {
+                        out_u8[3 * pid + 0] = encode_u8(r);
+                        out_u8[3 * pid + 1] = encode_u8(g);
+                        out_u8[3 * pid + 2] = encode_u8(b);
+                    }
+                    if (out_f32) {
+                        out_f32[3 * pid + 0] = r;
+                        out_f32[3 * pid + 1] = g;
+                        out_f32[3 * pid + 2] = b;
+                    }
+                }
             }
-            if (out_f32) {
-                out_f32[3 * pid + 0] = r;
-                out_f32[3 * pid + 1] = g;
-                out_f32[3 * pid + 2] = b;
-            }
-        }
-    }
 }
 
 int check_tile(int block_x, int block_y, int* sx, int* sy, const char* who)
@@ -212,7 +250,7 @@ int blend_impl(int block_x, int block_y, int width, int height,
     hipStream_t st = (hipStream_t)stream;
     const dim3 grid(tiles_x, tiles_y);
 #define FGS_LAUNCH_BLEND(SX, SY)                                                                        \
-    hipLaunchKernelGGL((blend_kernel<SX, SY>), grid, dim3(kBlendThreads), 0, st,                        \
+    hipLaunchKernelGGL((blend_kernel<SX, SY>), grid, dim3(kWave), 0, st,                                \
                        (const int2*)ranges, values_sorted, width, height, tiles_x,                      \
                        (const float2*)points_xy, (const float4*)rgb_depth, (const float4*)conic_opacity, \
                        bg[0], bg[1], bg[2], out_u8, out_f32)
