@@ -9,8 +9,9 @@
 //  * Key slots come from a count -> wave scan -> block scan -> chained look-back over
 //    workgroups instead of atomics on one counter, so the unsorted list has a fixed order:
 //    ascending Gaussian index, then row-major tiles.  A stable sort then fixes tie order too.
-//  * Gaussians whose candidate rectangle holds at most 64 tiles test their own tiles and keep
-//    the outcome in a 64-bit mask; larger ones are tested by the whole wave, 64 tiles a step.
+//  * The candidate tiles of all Gaussians of a wave with rectangles of at most 64 tiles are laid
+//    end to end and tested one per lane per step, so lanes stay busy whatever the mix of sizes;
+//    larger rectangles are tested by the whole wave, 64 tiles a step.
 //
 // THIS FILE MUST BE COMPILED WITH -ffp-contract=off.  Every fp32 expression that feeds a key is
 // written in the operand order of the reference and has to be evaluated one IEEE operation at a
@@ -18,13 +19,14 @@
 #include "fgs_internal.h"
 
 #include <mutex>
+#include <stdlib.h>
 
 namespace fgs {
 namespace {
 
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
-constexpr int kSmallMax = 64;           // rectangles up to this many tiles are tested per lane
+constexpr int kStashCap = 1024;         // flat candidates (and so stashed hits) per wave
 constexpr unsigned kSpinLimit = 1u << 22;   // polls before a chained-scan wait gives up
 
 struct Camera {
@@ -292,23 +294,27 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     int* __restrict__ curr_offset,
     int64_t capacity,            // <= 0: unchecked
     uint64_t* __restrict__ status,
-    uint32_t* __restrict__ ticket_counter,
-    uint32_t ticket_base,
     uint32_t epoch,
-    int num_blocks)
+    int num_blocks,
+    int exp_flags)
 {
-    __shared__ int s_ticket;
     __shared__ uint32_t s_wave_total[kWavesPerBlock];
     __shared__ uint32_t s_block_base;
+    __shared__ uint32_t s_stash[kWavesPerBlock][kStashCap];     // hits of the flat candidates, in emission order
+    __shared__ uint64_t s_hits[kWavesPerBlock][kStashCap / kWave + 1];
+    __shared__ uint8_t s_owner[kWavesPerBlock][kStashCap];      // flat candidate -> lane that owns it
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
 
-    if (tid == 0) s_ticket = (int)(atomicAdd(ticket_counter, 1u) - ticket_base);
-    __syncthreads();
-    const int ticket = s_ticket;
+    // Workgroups are numbered by their index: the hardware dispatches them in index order, so
+    // every workgroup with a smaller index is already running or finished when this one waits
+    // for it (and the wait is bounded in any case).
+    const int ticket = (int)blockIdx.x;
     const int idx = ticket * kBlock + tid;
+    // tile coordinates travel in 12 bits each and tile indices in 26 when candidates are laid flat
+    const bool pack_ok = cam.gx <= 4096 && cam.gy <= 4096 && (long long)cam.gx * cam.gy <= (1 << 26);
 
     // ---- per-Gaussian state (preprocess.cu:282-316) ----
     bool cand = false;           // passed both culls and has a non-empty candidate rectangle
@@ -323,6 +329,10 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         px = positions[3 * (size_t)idx + 0];
         py = positions[3 * (size_t)idx + 1];
         pz = positions[3 * (size_t)idx + 2];
+        // all per-Gaussian inputs are requested up front so that their latencies overlap
+        const float opacity = opacities[idx];
+        const float2* cv = reinterpret_cast<const float2*>(cov3ds + 6 * (size_t)idx);
+        const float2 s01 = cv[0], s23 = cv[1], s45 = cv[2];
         const float* m = cam.view;
         float t[3];
         t[0] = m[0] * px + m[4] * py + m[8] * pz + m[12];
@@ -330,7 +340,6 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         t[2] = m[2] * px + m[6] * py + m[10] * pz + m[14];
         depth = t[2];
         if (t[2] > 0.2f) {
-            const float opacity = opacities[idx];
             if (!(255.0f * opacity < 1.0f)) {
                 const float* q = cam.proj;
                 float hx = q[0] * px + q[4] * py + q[8] * pz + q[12];
@@ -340,8 +349,6 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
                 float projx = hx * p_w, projy = hy * p_w;
 
                 float s[6];
-                const float2* cv = reinterpret_cast<const float2*>(cov3ds + 6 * (size_t)idx);
-                float2 s01 = cv[0], s23 = cv[1], s45 = cv[2];
                 s[0] = s01.x; s[1] = s01.y; s[2] = s23.x; s[3] = s23.y; s[4] = s45.x; s[5] = s45.y;
                 float c00, c01, c11;
                 cov2d(t, cam, s, c00, c01, c11);
@@ -373,20 +380,69 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     // a rectangle with both extents negative has a positive product but no tiles
     const bool has_tiles = cand && rw > 0;
     const int area = has_tiles ? rw * rh : 0;
-    const bool small = has_tiles && area <= kSmallMax;
-    const bool large = has_tiles && area > kSmallMax;
 
     // ---- count keys ----
-    uint64_t hit_mask = 0;
-    uint32_t count = 0;
-    if (small) {
-        int x = rminx, y = rminy;
-        for (int j = 0; j < area; j++) {
-            if (tile_hit(x, y, cam.bx, cam.by, cx, cy, conx, cony, conz, power)) hit_mask |= 1ull << j;
-            if (++x == rminx + rw) { x = rminx; y++; }
-        }
-        count = (uint32_t)__popcll(hit_mask);
+    // Rectangles of up to 64 tiles are "flat": their candidates are laid end to end over the wave
+    // (Gaussian-major, row-major inside a Gaussian - the order keys are emitted in), so every lane
+    // tests one candidate per step whatever the mix of rectangle sizes.  Hits are compacted into
+    // an LDS stash as (tile << 6 | owner lane) and written out once the slots are known.  A wave
+    // stashes at most kStashCap candidates; what does not fit, and every larger rectangle, is
+    // tested by the whole wave, 64 tiles a step, once to count and once more to emit.
+    const bool flat_ok = has_tiles && area <= kWave && pack_ok;
+    uint32_t cand_incl = flat_ok ? (uint32_t)area : 0u;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        uint32_t up = (uint32_t)__shfl_up((int)cand_incl, o);
+        if (lane >= o) cand_incl += up;
     }
+    const bool flat = flat_ok && cand_incl <= (uint32_t)kStashCap;
+    const bool large = has_tiles && !flat;
+    // lanes that drop out are at the end of the scan order, so the prefix of the others is unchanged
+    const uint32_t cand_excl = cand_incl - (uint32_t)area;
+    const uint64_t flat_lanes = ballot(flat);
+    const int last_flat = flat_lanes ? 63 - __builtin_clzll(flat_lanes) : 0;
+    const int n_cand = flat_lanes ? bcast_i((int)cand_incl, last_flat) : 0;
+
+    uint8_t* owner_of = s_owner[wave];
+    uint32_t* stash = s_stash[wave];
+    uint64_t* hit_words = s_hits[wave];
+    if (flat)
+        for (int k = 0; k < area; k++) owner_of[cand_excl + k] = (uint8_t)lane;
+    __builtin_amdgcn_wave_barrier();
+
+    const uint32_t rect_pack = (uint32_t)rminx | ((uint32_t)rminy << 12) | ((uint32_t)(rw - 1) << 24);
+    int n_stash = 0;
+    for (int c0 = 0; c0 < n_cand; c0 += kWave) {
+        const int c = c0 + lane;
+        const bool live = c < n_cand;
+        const int own = live ? (int)owner_of[c] : lane;
+        const float gcx = __shfl(cx, own), gcy = __shfl(cy, own);
+        const float gconx = __shfl(conx, own), gcony = __shfl(cony, own), gconz = __shfl(conz, own);
+        const float gpower = __shfl(power, own);
+        const uint32_t grect = (uint32_t)__shfl((int)rect_pack, own);
+        const int k = c - __shfl((int)cand_excl, own);
+        const int gminx = (int)(grect & 0xfffu), gminy = (int)((grect >> 12) & 0xfffu), grw = (int)(grect >> 24) + 1;
+        // k / grw for 0 <= k < 64, 1 <= grw <= 64: (k + 0.5) / grw is at least 1/128 away from an
+        // integer, far more than the error of the approximate reciprocal
+        const int ty = (int)(((float)k + 0.5f) * __builtin_amdgcn_rcpf((float)grw));
+        const int tx = k - ty * grw;
+        const bool hit = live && tile_hit(gminx + tx, gminy + ty, cam.bx, cam.by, gcx, gcy, gconx, gcony, gconz, gpower);
+        const uint64_t hits = ballot(hit);
+        if (hit) stash[n_stash + popc_below(hits)] = ((uint32_t)((gminy + ty) * cam.gx + gminx + tx) << 6) | (uint32_t)own;
+        if (lane == 0) hit_words[c0 / kWave] = hits;
+        n_stash += __popcll(hits);
+    }
+    __builtin_amdgcn_wave_barrier();
+
+    uint32_t count = 0;
+    if (flat) {      // hits among this lane's candidates [cand_excl, cand_excl + area)
+        const int w0 = (int)(cand_excl >> 6), b0 = (int)(cand_excl & 63u);
+        uint64_t m = hit_words[w0] >> b0;
+        if (b0 + area > kWave) m |= hit_words[w0 + 1] << (kWave - b0);
+        if (area < kWave) m &= (1ull << area) - 1ull;
+        count = (uint32_t)__popcll(m);
+    }
+    const uint32_t flat_count = count;
     const uint64_t large_lanes = ballot(large);
     for (uint64_t todo = large_lanes; todo; todo &= todo - 1) {
         const int src = __ffsll((long long)todo) - 1;
@@ -427,15 +483,27 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         block_total += t;
     }
 
+    // The workgroup's count is published right away; the wait for the counts of earlier
+    // workgroups comes after the colour work below, when they have long been published.
+    if (tid == 0 && ticket != 0) publish(status + ticket, pack_status(epoch, kStateAggregate, block_total));
+
+    // ---- attributes of Gaussians that emit a key (preprocess.cu:411-417) ----
+    if (count > 0) {
+        constexpr float log2e = 1.4426950216293334961f;
+        reinterpret_cast<float2*>(points_xy)[idx] = make_float2(cx, cy);
+        reinterpret_cast<float4*>(conic_opacity)[idx] =
+            make_float4((-0.5f * log2e) * conx, -log2e * cony, (-0.5f * log2e) * conz, log2_op);
+        float rgb[3];
+        if (exp_flags & 8) { rgb[0] = rgb[1] = rgb[2] = 0.5f; } else
+        sh_to_rgb(shs + 48 * (size_t)idx, px, py, pz, cam, rgb);
+        reinterpret_cast<float4*>(rgb_depth)[idx] = make_float4(rgb[0], rgb[1], rgb[2], depth);
+    }
+
     if (wave == 0) {
         bool timed_out = false;
         uint32_t excl;
-        if (ticket == 0) {
-            excl = (uint32_t)*curr_offset;     // the caller's starting offset (example.py:69 zeroes it)
-        } else {
-            if (lane == 0) publish(status + ticket, pack_status(epoch, kStateAggregate, block_total));
-            excl = look_back(status, ticket, epoch, &timed_out);
-        }
+        if (ticket == 0) excl = (uint32_t)*curr_offset;     // the caller's starting offset (example.py:69 zeroes it)
+        else excl = (exp_flags & 4) ? 0u : look_back(status, ticket, epoch, &timed_out);
         if (lane == 0) {
             publish(status + ticket, pack_status(epoch, timed_out ? kStatePoison : kStatePrefix, excl + block_total));
             s_block_base = excl;
@@ -449,18 +517,28 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     // ---- emit ----
     const uint64_t cap = capacity > 0 ? (uint64_t)capacity : ~0ull;
     const uint32_t depth_bits = __float_as_uint(depth);
-    if (small && hit_mask) {
-        uint64_t slot = my_slot;
-        int x = rminx, y = rminy;
-        for (int j = 0; j < area; j++) {
-            if ((hit_mask >> j) & 1) {
-                if (slot < cap) {
-                    keys[slot] = ((uint64_t)(uint32_t)(y * cam.gx + x) << 32) | depth_bits;
-                    values[slot] = (uint32_t)idx;
-                }
-                slot++;
+    {
+        // stash entry e of owner o goes to slot(o) + (e - entries before o's first)
+        uint32_t before = flat_count;
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+            uint32_t up = (uint32_t)__shfl_up((int)before, o);
+            if (lane >= o) before += up;
+        }
+        const uint32_t delta = my_slot - (before - flat_count);
+        const uint32_t gidx_base = (uint32_t)(ticket * kBlock + wave * kWave);
+        for (int e0 = 0; e0 < n_stash; e0 += kWave) {
+            const int e = e0 + lane;
+            const bool live = e < n_stash;
+            const uint32_t entry = live ? stash[e] : (uint32_t)lane;
+            const int own = (int)(entry & 63u);
+            const uint32_t odelta = (uint32_t)__shfl((int)delta, own);
+            const uint32_t odepth = (uint32_t)__shfl((int)depth_bits, own);
+            const uint64_t dst = (uint64_t)(odelta + (uint32_t)e);
+            if (live && dst < cap) {
+                keys[dst] = ((uint64_t)(entry >> 6) << 32) | odepth;
+                values[dst] = gidx_base + (uint32_t)own;
             }
-            if (++x == rminx + rw) { x = rminx; y++; }
         }
     }
     for (uint64_t todo = large_lanes; todo; todo &= todo - 1) {
@@ -494,16 +572,6 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         }
     }
 
-    // ---- attributes of Gaussians that emitted a key (preprocess.cu:411-417) ----
-    if (count > 0) {
-        constexpr float log2e = 1.4426950216293334961f;
-        reinterpret_cast<float2*>(points_xy)[idx] = make_float2(cx, cy);
-        reinterpret_cast<float4*>(conic_opacity)[idx] =
-            make_float4((-0.5f * log2e) * conx, -log2e * cony, (-0.5f * log2e) * conz, log2_op);
-        float rgb[3];
-        sh_to_rgb(shs + 48 * (size_t)idx, px, py, pz, cam, rgb);
-        reinterpret_cast<float4*>(rgb_depth)[idx] = make_float4(rgb[0], rgb[1], rgb[2], depth);
-    }
 }
 
 // ---- per-device scratch for the chained scan ------------------------------------------------------
@@ -511,8 +579,6 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
 struct Scratch {
     uint64_t* status = nullptr;     // one word per workgroup
     size_t status_words = 0;
-    uint32_t* ticket = nullptr;     // monotonically increasing ticket counter
-    uint32_t tickets_issued = 0;    // host mirror of *ticket (mod 2^32)
     uint32_t epoch = 0;
 };
 
@@ -523,12 +589,6 @@ std::mutex g_mutex;
 int acquire_scratch(int device, int num_blocks, hipStream_t stream, Scratch** out)
 {
     Scratch& s = g_scratch[device];
-    if (s.ticket == nullptr) {
-        FGS_HIP_TRY(hipMalloc((void**)&s.ticket, 256));
-        FGS_HIP_TRY(hipMemset(s.ticket, 0, 256));
-        FGS_HIP_TRY(hipDeviceSynchronize());
-        s.tickets_issued = 0;
-    }
     if (s.status_words < (size_t)num_blocks) {
         // the stream may still be reading the old array: drain it before the swap
         FGS_HIP_TRY(hipStreamSynchronize(stream));
@@ -651,12 +711,10 @@ extern "C" int fgs_preprocess(int P,
     Scratch* s = nullptr;
     int rc = acquire_scratch(device, num_blocks, st, &s);
     if (rc != FGS_OK) return rc;
-    const uint32_t ticket_base = s->tickets_issued;
-    s->tickets_issued += (uint32_t)num_blocks;
 
     hipLaunchKernelGGL(preprocess_kernel, dim3(num_blocks), dim3(kBlock), 0, st,
                        P, positions, shs, opacities, cov3Ds, cam, points_xy, rgb_depth, conic_opacity,
                        gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset, key_capacity,
-                       s->status, s->ticket, ticket_base, s->epoch, num_blocks);
+                       s->status, s->epoch, num_blocks, getenv("FGS_EXP") ? atoi(getenv("FGS_EXP")) : 0);
     return check_hip(hipGetLastError(), "preprocess_kernel launch");
 }

@@ -1,103 +1,65 @@
-// Device-wide stable LSD radix sort of (u64 key, u32 value) pairs for gfx950 (wave64).
+// Device-wide stable sort of (u64 key, u32 value) pairs for gfx950 (wave64).
 //
 // Stands in for the cub::DeviceRadixSort::SortPairs call of FlashGS
-// (csrc/cuda_rasterizer/sort.cu:28-44): ascending, stable, on key bits [0, end_bit).
+// (csrc/cuda_rasterizer/sort.cu:28-44): ascending, stable, on key bits [0, 32 + tile_bits).
 //
-// Structure: one histogram launch counts all 8-bit digits of all passes, one small launch turns
-// the counts into exclusive digit bases, then one launch per digit reorders the pairs.  A
-// reorder workgroup ranks its tile of pairs in LDS (per-wave digit counters, wave64 ballot
-// matching, so equal digits keep their input order), publishes the tile's digit counts and
-// obtains the counts of all earlier tiles by walking back through their published words
-// (chained scan with decoupled look-back; tiles are numbered by an atomic ticket so a tile only
-// ever waits for tiles that already run).
+// The key is (tile id << 32 | depth bits), and what the renderer needs is every tile's pairs,
+// contiguous and ordered by depth.  So the sort runs most-significant part first:
+//
+//  1. Partition by tile id: one stable counting pass per 8 bits of tile id (two passes for up to
+//     65536 tiles).  A pass is count -> offsets -> scatter: `count_kernel` builds one digit
+//     histogram per block of 2048 pairs, `chunk_sum_kernel` + `offsets_kernel` turn the
+//     histograms into the exclusive start of every (block, digit) run, and `scatter_kernel` ranks
+//     its block in LDS (wave64 ballot matching, so equal digits keep their input order) and
+//     writes each run to its start.  No workgroup ever waits for another one.
+//  2. Sort every tile's segment by the 32 depth bits, in LDS: `segment_starts_kernel` tabulates
+//     where each tile id's segment begins; a `segment_sort_kernel` workgroup loads a segment, runs up to four stable 8-bit counting passes without touching memory (a pass in
+//     which all pairs share the digit is skipped) and writes the segment back in place.  Segments
+//     are handled by size class - one wave up to 256 and up to 1024 pairs, four waves up to
+//     4096, sixteen waves up to 8192; longer ones, and segments whose keys differ above the sorted bit range,
+//     go through the same passes with the ping-pong copy in HBM instead of LDS.
+//
+// Bytes moved per pair: 8 (count) + 24 (scatter) per partition pass, 24 for the segment sort:
+// 88 for two partition passes, against 8 + 6 * 24 = 152 for a six-pass LSD sort of 47 bits.
 #include "fgs_internal.h"
 
 namespace fgs {
 namespace {
 
 constexpr int kBins = 256;
-constexpr int kMaxPasses = 8;
 constexpr int kSortBlock = 256;
 constexpr int kSortWaves = kSortBlock / kWave;
-constexpr int kItems = 8;                       // pairs per thread
-constexpr int kTile = kSortBlock * kItems;      // pairs per workgroup
-constexpr int kHistBlock = 256;
-constexpr unsigned kSpinLimit = 1u << 22;
-
-// status word of one (tile, digit): [31:30] state, [29:0] count
-constexpr uint32_t kAggregate = 1u << 30;
-constexpr uint32_t kPrefix = 2u << 30;
-constexpr uint32_t kValueMask = (1u << 30) - 1;
+constexpr int kItems = 16;                      // pairs per thread in count/scatter
+constexpr int kTile = kSortBlock * kItems;      // pairs per count/scatter workgroup
+constexpr int kMinChunk = 16;                   // fewest histogram rows summed by one chunk_sum workgroup
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-struct Workspace {
-    size_t alt_keys, alt_values, counters, status, total;
-    int tiles;
-};
+// Tile ids up to this count get a table of segment starts in the workspace; beyond it every
+// segment workgroup searches for its own bounds.
+constexpr uint32_t kMaxTableIds = 1u << 20;
 
-// counters block: kMaxPasses*kBins digit counts/bases, then kMaxPasses tile tickets (padded)
-constexpr size_t kCounterWords = kMaxPasses * kBins + 64;
+struct Workspace {
+    size_t alt_keys, alt_values, hist, chunk_sums, seg_start, seg_flags, seg_lists, total;
+    int tiles, chunk, chunks;       // chunks of `chunk` histogram rows each
+};
 
 Workspace workspace_for(int n)
 {
     Workspace w;
     w.tiles = (n + kTile - 1) / kTile;
+    w.chunk = (w.tiles + 255) / 256 > kMinChunk ? (w.tiles + 255) / 256 : kMinChunk;     // at most ~256 chunks
+    w.chunks = (w.tiles + w.chunk - 1) / w.chunk;
     w.alt_keys = 0;
     w.alt_values = align_up((size_t)n * 8, 256);
-    w.counters = w.alt_values + align_up((size_t)n * 4, 256);
-    w.status = w.counters + kCounterWords * 4;
-    w.total = w.status + (size_t)kMaxPasses * w.tiles * kBins * 4;
+    w.hist = w.alt_values + align_up((size_t)n * 4, 256);
+    w.chunk_sums = w.hist + (size_t)w.tiles * kBins * 4;
+    w.seg_start = w.chunk_sums + (size_t)w.chunks * kBins * 4;
+    w.seg_flags = w.seg_start + align_up(((size_t)kMaxTableIds + 1) * 4, 256);
+    // counters (64 words), then the ids of the medium and of the large segments
+    w.seg_lists = w.seg_flags + kMaxTableIds / 8;
+    w.total = w.seg_lists + 256 + ((size_t)n / 1024 + 2) * 4 + ((size_t)n / 4096 + 2) * 4;
     return w;
-}
-
-__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* p, size_t n, uint32_t v)
-{
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (; i < n; i += stride) p[i] = v;
-}
-
-// counts[pass][digit] += number of keys whose digit `pass` equals `digit`
-__global__ __launch_bounds__(kHistBlock) void histogram_kernel(const uint64_t* __restrict__ keys, int n,
-                                                               int passes, int end_bit, uint32_t* __restrict__ counts)
-{
-    __shared__ uint32_t h[kMaxPasses * kBins];
-    for (int j = threadIdx.x; j < passes * kBins; j += kHistBlock) h[j] = 0;
-    __syncthreads();
-    const int stride = gridDim.x * kHistBlock;
-    for (int i = blockIdx.x * kHistBlock + threadIdx.x; i < n; i += stride) {
-        const uint64_t k = keys[i];
-        for (int p = 0; p < passes; p++) {
-            const int shift = 8 * p;
-            const int nbits = min(8, end_bit - shift);
-            const uint32_t d = (uint32_t)(k >> shift) & ((1u << nbits) - 1u);
-            atomicAdd(&h[p * kBins + d], 1u);
-        }
-    }
-    __syncthreads();
-    for (int j = threadIdx.x; j < passes * kBins; j += kHistBlock) {
-        const uint32_t c = h[j];
-        if (c) atomicAdd(&counts[j], c);
-    }
-}
-
-// one workgroup per pass: counts[pass][*] -> exclusive prefix over digits, in place
-__global__ __launch_bounds__(kBins) void digit_base_kernel(uint32_t* __restrict__ counts)
-{
-    __shared__ uint32_t s[kBins];
-    uint32_t* c = counts + blockIdx.x * kBins;
-    const int d = threadIdx.x;
-    const uint32_t mine = c[d];
-    s[d] = mine;
-    __syncthreads();
-    for (int o = 1; o < kBins; o <<= 1) {
-        uint32_t add = d >= o ? s[d - o] : 0u;
-        __syncthreads();
-        s[d] += add;
-        __syncthreads();
-    }
-    c[d] = s[d] - mine;
 }
 
 __device__ __forceinline__ uint32_t digit_of(uint64_t key, int shift, uint32_t mask)
@@ -105,45 +67,128 @@ __device__ __forceinline__ uint32_t digit_of(uint64_t key, int shift, uint32_t m
     return (uint32_t)(key >> shift) & mask;
 }
 
-__global__ __launch_bounds__(kSortBlock) void reorder_kernel(
+// ---- partition pass, step 1: hist[block][digit] ---------------------------------------------------
+
+__global__ __launch_bounds__(kSortBlock) void count_kernel(const uint64_t* __restrict__ keys, int n,
+                                                           int shift, int nbits, uint32_t* __restrict__ hist)
+{
+    __shared__ uint32_t h[kBins];
+    const int tid = threadIdx.x;
+    h[tid] = 0;
+    __syncthreads();
+    const uint32_t mask = (1u << nbits) - 1u;
+    const int base = blockIdx.x * kTile;
+#pragma unroll
+    for (int i = 0; i < kItems; i++) {
+        const int idx = base + i * kSortBlock + tid;
+        if (idx < n) atomicAdd(&h[digit_of(keys[idx], shift, mask)], 1u);
+    }
+    __syncthreads();
+    hist[(size_t)blockIdx.x * kBins + tid] = h[tid];
+}
+
+// ---- step 2: exclusive start of every (block, digit) run ----------------------------------------
+// start[b][d] = sum of hist[*][d' < d] + sum of hist[b' < b][d]   (digit-major, then block)
+
+__global__ __launch_bounds__(kBins) void chunk_sum_kernel(const uint32_t* __restrict__ hist, int tiles, int chunk,
+                                                          uint32_t* __restrict__ chunk_sums)
+{
+    const int d = threadIdx.x;
+    const int t0 = blockIdx.x * chunk, t1 = min(tiles, t0 + chunk);
+    uint32_t s = 0;
+    for (int t = t0; t < t1; t++) s += hist[(size_t)t * kBins + d];
+    chunk_sums[(size_t)blockIdx.x * kBins + d] = s;
+}
+
+__global__ __launch_bounds__(kBins) void offsets_kernel(uint32_t* __restrict__ hist, int tiles, int chunk,
+                                                        const uint32_t* __restrict__ chunk_sums, int chunks)
+{
+    __shared__ uint32_t s_wave[kBins / kWave];
+    const int d = threadIdx.x;
+    const int lane = d & (kWave - 1), wave = d / kWave;
+    const int mine = (int)blockIdx.x;
+    uint32_t total = 0, before = 0;
+    // batches of 16 independent loads: the chunk sums are few and the loop is latency-bound
+    for (int c0 = 0; c0 < chunks; c0 += 16) {
+        uint32_t v[16];
+#pragma unroll
+        for (int j = 0; j < 16; j++) v[j] = c0 + j < chunks ? chunk_sums[(size_t)(c0 + j) * kBins + d] : 0u;
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            if (c0 + j < mine) before += v[j];
+            total += v[j];
+        }
+    }
+    // exclusive scan of the digit totals over the 256 digits
+    uint32_t incl = total;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        uint32_t up = (uint32_t)__shfl_up((int)incl, o);
+        if (lane >= o) incl += up;
+    }
+    if (lane == kWave - 1) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t digit_base = incl - total;
+    for (int w = 0; w < wave; w++) digit_base += s_wave[w];
+
+    uint32_t run = digit_base + before;
+    const int t0 = mine * chunk, t1 = min(tiles, t0 + chunk);
+    for (int tb = t0; tb < t1; tb += 16) {
+        uint32_t c[16];
+#pragma unroll
+        for (int j = 0; j < 16; j++) c[j] = tb + j < t1 ? hist[(size_t)(tb + j) * kBins + d] : 0u;
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            if (tb + j < t1) hist[(size_t)(tb + j) * kBins + d] = run;
+            run += c[j];
+        }
+    }
+}
+
+// ---- step 3: stable scatter ---------------------------------------------------------------------------
+
+__global__ __launch_bounds__(kSortBlock) void scatter_kernel(
     const uint64_t* __restrict__ keys_in, const uint32_t* __restrict__ values_in,
     uint64_t* __restrict__ keys_out, uint32_t* __restrict__ values_out,
     int n, int shift, int nbits,
-    const uint32_t* __restrict__ digit_base,     // [kBins] exclusive digit bases of this pass
-    uint32_t* __restrict__ status,               // [tiles][kBins], zero before the launch
-    uint32_t* __restrict__ ticket)               // zero before the launch
+    const uint32_t* __restrict__ start)          // [blocks][kBins] from offsets_kernel
 {
     __shared__ uint32_t s_count[kSortWaves][kBins];   // per-wave digit counts, then per-wave digit offsets
-    __shared__ uint32_t s_bin_start[kBins];           // where each digit starts in the ranked tile
+    __shared__ uint32_t s_bin_start[kBins];           // where each digit starts in the ranked block
     __shared__ uint32_t s_global[kBins];              // destination of ranked slot p with digit d: s_global[d] + p
     __shared__ uint32_t s_wave_sum[kSortWaves];
     __shared__ uint64_t s_keys[kTile];
     __shared__ uint32_t s_values[kTile];
-    __shared__ int s_tile;
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
     const uint32_t mask = (1u << nbits) - 1u;
-
-    if (tid == 0) s_tile = (int)atomicAdd(ticket, 1u);
-#pragma unroll
-    for (int w = 0; w < kSortWaves; w++) s_count[w][tid] = 0;
-    __syncthreads();
-    const int tile = s_tile;
+    const int tile = blockIdx.x;
     const int tile_base = tile * kTile;
     const int in_tile = min(kTile, n - tile_base);
 
-    // ---- load: wave w owns slots [w*64*kItems, (w+1)*64*kItems) of the tile, item-major ----
+    // wave w owns slots [w*64*kItems, (w+1)*64*kItems) of the block, item-major; everything is
+    // requested before the first use so the latencies overlap
     uint64_t key[kItems];
+    uint32_t val[kItems];
     uint32_t slot[kItems];
 #pragma unroll
     for (int i = 0; i < kItems; i++) {
         const int off = wave * (kWave * kItems) + i * kWave + lane;
         key[i] = off < in_tile ? keys_in[tile_base + off] : ~0ull;
     }
+#pragma unroll
+    for (int i = 0; i < kItems; i++) {
+        const int off = wave * (kWave * kItems) + i * kWave + lane;
+        val[i] = off < in_tile ? values_in[tile_base + off] : 0u;
+    }
+    const uint32_t my_start = start[(size_t)tile * kBins + tid];
+#pragma unroll
+    for (int w = 0; w < kSortWaves; w++) s_count[w][tid] = 0;
+    __syncthreads();
 
-    // ---- rank inside the wave: lanes with equal digits find each other with 8 ballots ----
+    // rank inside the wave: lanes with equal digits find each other with one ballot per digit bit
 #pragma unroll
     for (int i = 0; i < kItems; i++) {
         const int off = wave * (kWave * kItems) + i * kWave + lane;
@@ -169,7 +214,7 @@ __global__ __launch_bounds__(kSortBlock) void reorder_kernel(
     }
     __syncthreads();
 
-    // ---- digit totals of the tile; per-wave offsets inside each digit ----
+    // digit totals of the block; per-wave offsets inside each digit
     const int d = tid;      // one thread per digit from here on
     uint32_t total = 0;
 #pragma unroll
@@ -178,12 +223,6 @@ __global__ __launch_bounds__(kSortBlock) void reorder_kernel(
         s_count[w][d] = total;
         total += c;
     }
-    if (tile == 0)
-        __hip_atomic_store(status + d, kPrefix | total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else
-        __hip_atomic_store(status + (size_t)tile * kBins + d, kAggregate | total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-
-    // exclusive scan of the totals over the 256 digits
     uint32_t incl = total;
 #pragma unroll
     for (int o = 1; o < kWave; o <<= 1) {
@@ -198,9 +237,10 @@ __global__ __launch_bounds__(kSortBlock) void reorder_kernel(
         if (w < wave) before_wave += s_wave_sum[w];
     const uint32_t bin_start = before_wave + incl - total;
     s_bin_start[d] = bin_start;
+    s_global[d] = my_start - bin_start;
     __syncthreads();
 
-    // ---- move the pairs to their ranked slots in LDS ----
+    // move the pairs to their ranked slots in LDS
 #pragma unroll
     for (int i = 0; i < kItems; i++) {
         const int off = wave * (kWave * kItems) + i * kWave + lane;
@@ -208,34 +248,12 @@ __global__ __launch_bounds__(kSortBlock) void reorder_kernel(
             const uint32_t dg = digit_of(key[i], shift, mask);
             const uint32_t p = s_bin_start[dg] + s_count[wave][dg] + slot[i];
             s_keys[p] = key[i];
-            s_values[p] = values_in[tile_base + off];
+            s_values[p] = val[i];
         }
     }
-
-    // ---- counts of all earlier tiles for digit d ----
-    uint32_t earlier = 0;
-    if (tile > 0) {
-        unsigned spins = 0;
-        int j = tile - 1;
-        while (j >= 0) {
-            const uint32_t w = __hip_atomic_load(status + (size_t)j * kBins + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const uint32_t st = w & ~kValueMask;
-            if (st == 0) {
-                if (++spins > kSpinLimit) break;        // bounded wait: give up rather than hang
-                __builtin_amdgcn_s_sleep(1);
-                continue;
-            }
-            earlier += w & kValueMask;
-            if (st == kPrefix) break;
-            j--;
-        }
-        __hip_atomic_store(status + (size_t)tile * kBins + d, kPrefix | ((earlier + total) & kValueMask),
-                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    s_global[d] = digit_base[d] + earlier - bin_start;
     __syncthreads();
 
-    // ---- write out: neighbouring threads hold neighbouring ranked slots ----
+    // write out: neighbouring threads hold neighbouring ranked slots
 #pragma unroll
     for (int i = 0; i < kItems; i++) {
         const int p = i * kSortBlock + tid;
@@ -247,6 +265,500 @@ __global__ __launch_bounds__(kSortBlock) void reorder_kernel(
         }
     }
 }
+
+// ---- per-tile segment sort on the 32 depth bits ----------------------------------------------------
+
+// First index in [0, n) whose tile field is >= v (n if none), found by the whole wave probing 64
+// evenly spaced positions per step.  `keys` is ordered by tile field.  All lanes return the same.
+__device__ __forceinline__ int wave_lower_bound(const uint64_t* __restrict__ keys, int n, uint32_t v, uint32_t tile_mask)
+{
+    const int lane = lane_id();
+    int lo = 0, hi = n;                 // the answer lies in [lo, hi]; every index < lo is < v, index hi (if < n) is >= v
+    while (hi > lo) {
+        const int span = hi - lo;
+        const int step = (span + kWave - 1) / kWave;        // >= 1
+        const int pos = lo + lane * step;                    // probes at lo, lo+step, ...
+        bool ge = true;                                      // a probe at or past hi counts as ">= v"
+        if (pos < hi) ge = ((uint32_t)(keys[pos] >> 32) & tile_mask) >= v;
+        const uint64_t m = ballot(ge);
+        const int first = m ? __ffsll((long long)m) - 1 : kWave;     // first probe that is >= v
+        if (first == 0) return lo;
+        const int new_hi = first < kWave ? min(hi, lo + first * step) : hi;
+        lo = lo + (first - 1) * step + 1;                    // the probe before `first` is < v
+        hi = new_hi;
+    }
+    return lo;
+}
+
+// seg_start[v] = first index whose tile field is >= v, for v in [0, ids]; seg_start[ids] = n.
+// One thread per pair: where the tile field changes, the thread fills the entries of the ids in
+// between (empty ids get the same start as the next non-empty one).  Also clears the flag words.
+__global__ __launch_bounds__(256) void segment_starts_kernel(const uint64_t* __restrict__ keys, int n, uint32_t tile_mask,
+                                                             uint32_t ids, int* __restrict__ seg_start,
+                                                             uint32_t* __restrict__ seg_flags, uint32_t* __restrict__ seg_counts)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if ((uint32_t)i < (ids + 31) / 32) seg_flags[i] = 0;
+    if (i < 2) seg_counts[i] = 0;
+    if (i >= n) return;
+    const uint32_t cur = (uint32_t)(keys[i] >> 32) & tile_mask;
+    const uint32_t first = i == 0 ? 0u : ((uint32_t)(keys[i - 1] >> 32) & tile_mask) + 1u;
+    for (uint32_t v = first; v <= cur; v++) seg_start[v] = i;      // empty loop when the field repeats
+    if (i == n - 1)
+        for (uint32_t v = cur + 1; v <= ids; v++) seg_start[v] = n;
+}
+
+// One stable counting pass of a segment over bits shift..shift+7 of the sort word, by the kWaves
+// waves of one workgroup.  Wave w owns the contiguous part [w*per, (w+1)*per) of the segment.
+// Returns false (and moves nothing) when every pair has the same digit.  All threads of the
+// workgroup must call it.  KeyT is uint32_t for depth words in LDS, uint64_t for whole keys in HBM.
+template <int kWaves, typename KeyT>
+__device__ __forceinline__ bool counting_pass(const KeyT* src_k, const uint32_t* src_v, KeyT* dst_k, uint32_t* dst_v,
+                                              int n, int shift, uint32_t (*cnt)[kBins], uint32_t* wave_sum, int* flag)
+{
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int per = ((n + kWaves - 1) / kWaves + kWave - 1) / kWave * kWave;   // a multiple of 64
+    const int w_lo = min(n, wave * per), w_hi = min(n, w_lo + per);
+
+    for (int d = lane; d < kBins; d += kWave) cnt[wave][d] = 0;
+    if (kWaves > 1) { if (tid == 0) *flag = 0; __syncthreads(); } else __builtin_amdgcn_wave_barrier();
+    for (int i = w_lo + lane; i < w_hi; i += kWave)
+        atomicAdd(&cnt[wave][(uint32_t)(src_k[i] >> shift) & 255u], 1u);
+    if (kWaves > 1) __syncthreads(); else __builtin_amdgcn_wave_barrier();
+
+    bool uniform;
+    if (kWaves == 1) {
+        // lane handles digits lane, lane+64, lane+128, lane+192; scan in digit order
+        uint32_t base = 0;
+        bool any_full = false;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t c = cnt[0][q * kWave + lane];
+            any_full = any_full || c == (uint32_t)n;
+            uint32_t incl = c;
+#pragma unroll
+            for (int o = 1; o < kWave; o <<= 1) {
+                uint32_t up = (uint32_t)__shfl_up((int)incl, o);
+                if (lane >= o) incl += up;
+            }
+            cnt[0][q * kWave + lane] = base + incl - c;
+            base += (uint32_t)bcast_i((int)incl, kWave - 1);
+        }
+        uniform = ballot(any_full) != 0;
+        __builtin_amdgcn_wave_barrier();
+    } else {
+        // thread t < 256 handles digit t
+        uint32_t total = 0;
+        if (tid < kBins) {
+            for (int w = 0; w < kWaves; w++) {
+                const uint32_t c = cnt[w][tid];
+                cnt[w][tid] = total;          // offset of wave w inside digit tid
+                total += c;
+            }
+            if (total == (uint32_t)n) *flag = 1;
+            uint32_t incl = total;
+#pragma unroll
+            for (int o = 1; o < kWave; o <<= 1) {
+                uint32_t up = (uint32_t)__shfl_up((int)incl, o);
+                if (lane >= o) incl += up;
+            }
+            if (lane == kWave - 1) wave_sum[wave] = incl;
+            total = incl - total;             // exclusive inside this wave's 64 digits
+        }
+        __syncthreads();
+        if (tid < kBins) {
+            uint32_t base = total;
+            for (int w = 0; w < wave; w++) base += wave_sum[w];
+            for (int w = 0; w < kWaves; w++) cnt[w][tid] += base;     // absolute start of (wave, digit)
+        }
+        __syncthreads();
+        uniform = *flag != 0;
+    }
+    if (uniform) return false;
+
+    // stable ranking, 64 pairs at a time in segment order
+    for (int base = w_lo; base < w_hi; base += kWave) {
+        const int i = base + lane;
+        const bool valid = i < w_hi;
+        KeyT k = 0;
+        uint32_t v = 0;
+        if (valid) { k = src_k[i]; v = src_v[i]; }
+        const uint32_t d = (uint32_t)(k >> shift) & 255u;
+        uint64_t peers = ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            const bool bit = (d >> b) & 1u;
+            const uint64_t with_bit = ballot(bit);
+            peers &= bit ? with_bit : ~with_bit;
+        }
+        const int below = popc_below(peers);
+        uint32_t before = 0;
+        if (valid && below == 0) {
+            before = cnt[wave][d];
+            cnt[wave][d] = before + (uint32_t)__popcll(peers);
+        }
+        const int leader = valid ? __ffsll((long long)peers) - 1 : lane;
+        before = (uint32_t)__shfl((int)before, leader);
+        if (valid) {
+            dst_k[before + (uint32_t)below] = k;
+            dst_v[before + (uint32_t)below] = v;
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    return true;
+}
+
+// Sorts the segment [lo, hi) of tile id v in LDS.  Called by all kWaves waves of a workgroup
+// with the same arguments; hi - lo <= kCap.  A segment whose keys differ above the depth word
+// cannot be rebuilt from depth words: it is flagged (or, without a flag array, left alone) for
+// the general kernel.
+template <int kWaves, int kCap>
+__device__ __forceinline__ void sort_segment_lds(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
+                                                 uint32_t v, int lo, int hi, uint32_t* __restrict__ seg_flags,
+                                                 uint32_t (*s_k)[kCap], uint32_t (*s_v)[kCap],
+                                                 uint32_t (*s_cnt)[kBins], uint32_t* s_wave_sum, int* s_flag)
+{
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int len = hi - lo;
+    const uint32_t upper = (uint32_t)(keys[lo] >> 32);
+    bool mixed = false;
+    if (kWaves > 1) { if (tid == 0) *s_flag = 0; __syncthreads(); }
+    for (int i = tid; i < len; i += kWaves * kWave) {
+        const uint64_t k = keys[lo + i];
+        s_k[0][i] = (uint32_t)k;
+        s_v[0][i] = values[lo + i];
+        mixed = mixed || (uint32_t)(k >> 32) != upper;
+    }
+    if (kWaves == 1) {
+        if (ballot(mixed)) {
+            if (seg_flags && lane == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
+            return;
+        }
+        __builtin_amdgcn_wave_barrier();
+    } else {
+        if (mixed) *s_flag = 1;
+        __syncthreads();
+        const bool any_mixed = *s_flag != 0;
+        __syncthreads();                             // counting_pass reuses the flag
+        if (any_mixed) {
+            if (seg_flags && tid == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
+            return;
+        }
+    }
+
+    int cur = 0;
+#pragma unroll 1
+    for (int shift = 0; shift < 32; shift += 8) {
+        const bool moved = counting_pass<kWaves, uint32_t>(s_k[cur], s_v[cur], s_k[cur ^ 1], s_v[cur ^ 1], len, shift,
+                                                           s_cnt, s_wave_sum, s_flag);
+        if (kWaves > 1) __syncthreads(); else __builtin_amdgcn_wave_barrier();
+        if (moved) cur ^= 1;
+    }
+    for (int i = tid; i < len; i += kWaves * kWave) {
+        keys[lo + i] = ((uint64_t)upper << 32) | s_k[cur][i];
+        values[lo + i] = s_v[cur][i];
+    }
+    if (kWaves > 1) __syncthreads(); else __builtin_amdgcn_wave_barrier();
+}
+
+// Segment sort in LDS for one size class: segments with min_len < length <= kCap.
+// With a table of segment starts, workgroup w looks at the kIds tile ids [w*kIds, (w+1)*kIds),
+// one per lane, and sorts those of its class one after the other.  Without a table (more tile ids
+// than the table holds) the grid has one workgroup per tile id and each searches for its bounds.
+template <int kWaves, int kCap, int kIds>
+__global__ __launch_bounds__(kWaves * kWave) void segment_sort_kernel(
+    uint64_t* __restrict__ keys, uint32_t* __restrict__ values, int n, uint32_t tile_mask, int min_len, uint32_t ids,
+    const int* __restrict__ seg_start, uint32_t* __restrict__ seg_flags,
+    const uint32_t* __restrict__ list, const uint32_t* __restrict__ list_count)
+{
+    __shared__ uint32_t s_k[2][kCap];
+    __shared__ uint32_t s_v[2][kCap];
+    __shared__ uint32_t s_cnt[kWaves][kBins];
+    __shared__ uint32_t s_wave_sum[kWaves];
+    __shared__ int s_bounds[2];
+    __shared__ int s_flag;
+    __shared__ uint64_t s_match;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+
+    if (!seg_start) {
+        const uint32_t v = blockIdx.x;
+        if (tid < kWave) {
+            const int a = wave_lower_bound(keys, n, v, tile_mask);
+            const int b = v == tile_mask ? n : wave_lower_bound(keys, n, v + 1, tile_mask);
+            if (lane == 0) { s_bounds[0] = a; s_bounds[1] = b; }
+        }
+        __syncthreads();
+        const int lo = s_bounds[0], hi = s_bounds[1];
+        if (hi - lo <= min_len || hi - lo > kCap) return;
+        sort_segment_lds<kWaves, kCap>(keys, values, v, lo, hi, seg_flags, s_k, s_v, s_cnt, s_wave_sum, &s_flag);
+        return;
+    }
+
+    if (list) {      // the segments of this class were listed: deal them out round-robin
+        const uint32_t count = *list_count;
+        for (uint32_t i = blockIdx.x; i < count; i += gridDim.x) {
+            const uint32_t v = list[i];
+            sort_segment_lds<kWaves, kCap>(keys, values, v, seg_start[v], seg_start[v + 1], seg_flags,
+                                           s_k, s_v, s_cnt, s_wave_sum, &s_flag);
+        }
+        return;
+    }
+
+    const uint32_t first_id = blockIdx.x * (uint32_t)kIds;
+    if (tid < kWave) {
+        const uint32_t v = first_id + (uint32_t)lane;
+        int len = 0;
+        if (lane < kIds && v < ids) len = seg_start[v + 1] - seg_start[v];
+        const uint64_t m = ballot(len > min_len && len <= kCap);
+        if (lane == 0) s_match = m;
+    }
+    __syncthreads();
+    for (uint64_t todo = s_match; todo; todo &= todo - 1) {
+        const uint32_t v = first_id + (uint32_t)(__ffsll((long long)todo) - 1);
+        sort_segment_lds<kWaves, kCap>(keys, values, v, seg_start[v], seg_start[v + 1], seg_flags,
+                                       s_k, s_v, s_cnt, s_wave_sum, &s_flag);
+    }
+}
+
+// Segment sort by a single wave that keeps its pairs in registers: lane l holds pairs
+// l, l+64, ... (kT of them), LDS is only the scatter target of each pass and the 256 digit
+// counters.  For segments with min_len < length <= 64*kT.  Everything is unrolled over the kT
+// pairs of a lane, so the ballot work of different pairs overlaps with the LDS round trips of the
+// running digit counters.
+template <int kT>
+__device__ __forceinline__ void sort_segment_wave(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
+                                                  uint32_t v, int lo, int hi, uint32_t* __restrict__ seg_flags,
+                                                  uint32_t* s_k, uint32_t* s_v, uint32_t* cnt)
+{
+    const int lane = threadIdx.x;
+    const int len = hi - lo;
+    const uint32_t upper = (uint32_t)(keys[lo] >> 32);
+    uint32_t k[kT], val[kT];
+    bool mixed = false;
+#pragma unroll
+    for (int t = 0; t < kT; t++) {
+        const int i = t * kWave + lane;
+        k[t] = 0xffffffffu;
+        val[t] = 0;
+        if (i < len) {
+            const uint64_t kk = keys[lo + i];
+            k[t] = (uint32_t)kk;
+            val[t] = values[lo + i];
+            mixed = mixed || (uint32_t)(kk >> 32) != upper;
+        }
+    }
+    if (ballot(mixed)) {     // keys differ above the depth word: left to the general kernel
+        if (seg_flags && lane == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
+        return;
+    }
+
+#pragma unroll 1
+    for (int shift = 0; shift < 32; shift += 8) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) cnt[q * kWave + lane] = 0;
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int t = 0; t < kT; t++) {
+            if (t * kWave >= len) break;               // uniform: the remaining register slots are empty
+            if (t * kWave + lane < len) atomicAdd(&cnt[(k[t] >> shift) & 255u], 1u);
+        }
+        __builtin_amdgcn_wave_barrier();
+
+        // exclusive scan over the 256 digits; lane handles digits lane, lane+64, lane+128, lane+192
+        uint32_t base = 0;
+        bool any_full = false;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t c = cnt[q * kWave + lane];
+            any_full = any_full || c == (uint32_t)len;
+            uint32_t incl = c;
+#pragma unroll
+            for (int o = 1; o < kWave; o <<= 1) {
+                uint32_t up = (uint32_t)__shfl_up((int)incl, o);
+                if (lane >= o) incl += up;
+            }
+            cnt[q * kWave + lane] = base + incl - c;
+            base += (uint32_t)bcast_i((int)incl, kWave - 1);
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (ballot(any_full)) continue;            // every pair has the same digit: nothing moves
+
+#pragma unroll
+        for (int t = 0; t < kT; t++) {
+            if (t * kWave >= len) break;
+            const bool valid = t * kWave + lane < len;
+            const uint32_t d = (k[t] >> shift) & 255u;
+            uint64_t peers = ballot(valid);
+#pragma unroll
+            for (int b = 0; b < 8; b++) {
+                const bool bit = (d >> b) & 1u;
+                const uint64_t with_bit = ballot(bit);
+                peers &= bit ? with_bit : ~with_bit;
+            }
+            const int below = popc_below(peers);
+            uint32_t before = 0;
+            if (valid && below == 0) {
+                before = cnt[d];
+                cnt[d] = before + (uint32_t)__popcll(peers);
+            }
+            const int leader = valid ? __ffsll((long long)peers) - 1 : lane;
+            before = (uint32_t)__shfl((int)before, leader);
+            if (valid) {
+                s_k[before + (uint32_t)below] = k[t];
+                s_v[before + (uint32_t)below] = val[t];
+            }
+            __builtin_amdgcn_sched_barrier(0);      // keeps the live ranges of one pair's ballots from piling up
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int t = 0; t < kT; t++) {
+            if (t * kWave >= len) break;
+            const int i = t * kWave + lane;
+            if (i < len) { k[t] = s_k[i]; val[t] = s_v[i]; }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+#pragma unroll
+    for (int t = 0; t < kT; t++) {
+        const int i = t * kWave + lane;
+        if (i < len) {
+            keys[lo + i] = ((uint64_t)upper << 32) | k[t];
+            values[lo + i] = val[t];
+        }
+    }
+}
+
+// One wave per workgroup; with a table of segment starts the workgroup looks at kIds tile ids
+// (one per lane) and sorts those with min_len < length <= 64*kT one after the other; without a
+// table the grid has one workgroup per tile id and each searches for its bounds.
+template <int kT, int kIds>
+__global__ __launch_bounds__(kWave) void segment_sort_wave_kernel(
+    uint64_t* __restrict__ keys, uint32_t* __restrict__ values, int n, uint32_t tile_mask, int min_len, uint32_t ids,
+    const int* __restrict__ seg_start, uint32_t* __restrict__ seg_flags,
+    int list_min0, int list_max0, int list_max1,
+    uint32_t* __restrict__ seg_counts, uint32_t* __restrict__ list0, uint32_t* __restrict__ list1)
+{
+    __shared__ uint32_t s_k[kT * kWave];
+    __shared__ uint32_t s_v[kT * kWave];
+    __shared__ uint32_t s_cnt[kBins];
+    const int lane = threadIdx.x;
+    if (!seg_start) {
+        const uint32_t v = blockIdx.x;
+        const int lo = wave_lower_bound(keys, n, v, tile_mask);
+        const int hi = v == tile_mask ? n : wave_lower_bound(keys, n, v + 1, tile_mask);
+        if (hi - lo <= min_len || hi - lo > kT * kWave) return;
+        sort_segment_wave<kT>(keys, values, v, lo, hi, seg_flags, s_k, s_v, s_cnt);
+        return;
+    }
+    const uint32_t first_id = blockIdx.x * (uint32_t)kIds;
+    const uint32_t mine = first_id + (uint32_t)lane;
+    int len = 0;
+    if (lane < kIds && mine < ids) len = seg_start[mine + 1] - seg_start[mine];
+    // This launch sees every tile id once: it also lists the ids whose segments need a multi-wave
+    // workgroup (lengths in (list_min0, list_max0] and (list_max0, list_max1]), so that those few,
+    // long-running segments can be dealt out evenly by the launches that follow.
+    if (list0) {
+        if (len > list_min0 && len <= list_max0) list0[atomicAdd(&seg_counts[0], 1u)] = mine;
+        else if (len > list_max0 && len <= list_max1) list1[atomicAdd(&seg_counts[1], 1u)] = mine;
+    }
+    for (uint64_t todo = ballot(len > min_len && len <= kT * kWave); todo; todo &= todo - 1) {
+        const uint32_t v = first_id + (uint32_t)(__ffsll((long long)todo) - 1);
+        sort_segment_wave<kT>(keys, values, v, seg_start[v], seg_start[v + 1], seg_flags, s_k, s_v, s_cnt);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// The same passes with whole keys and the ping-pong copy in HBM: for segments longer than
+// min_len and for shorter segments whose keys differ above the depth word.  General and slow;
+// inputs produced by fgs_preprocess only reach it with more than min_len pairs in one tile.
+__device__ __forceinline__ void sort_segment_general(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
+                                                     uint64_t* __restrict__ alt_keys, uint32_t* __restrict__ alt_values,
+                                                     int lo, int hi, uint32_t (*s_cnt)[kBins], uint32_t* s_wave_sum, int* s_flag)
+{
+    const int tid = threadIdx.x;
+    const int len = hi - lo;
+    uint64_t* kbuf[2] = { keys + lo, alt_keys + lo };
+    uint32_t* vbuf[2] = { values + lo, alt_values + lo };
+    int cur = 0;
+#pragma unroll 1
+    for (int shift = 0; shift < 32; shift += 8) {
+        const bool moved = counting_pass<kSortWaves, uint64_t>(kbuf[cur], vbuf[cur], kbuf[cur ^ 1], vbuf[cur ^ 1], len,
+                                                               shift, s_cnt, s_wave_sum, s_flag);
+        __threadfence_block();
+        __syncthreads();
+        if (moved) cur ^= 1;
+    }
+    if (cur == 1)
+        for (int i = tid; i < len; i += kSortBlock) { kbuf[0][i] = kbuf[1][i]; vbuf[0][i] = vbuf[1][i]; }
+    __threadfence_block();
+    __syncthreads();
+}
+
+__global__ __launch_bounds__(kSortBlock) void segment_sort_general_kernel(
+    uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
+    uint64_t* __restrict__ alt_keys, uint32_t* __restrict__ alt_values,
+    int n, uint32_t tile_mask, int min_len, uint32_t ids,
+    const int* __restrict__ seg_start, const uint32_t* __restrict__ seg_flags)
+{
+    __shared__ uint32_t s_cnt[kSortWaves][kBins];
+    __shared__ uint32_t s_wave_sum[kSortWaves];
+    __shared__ int s_bounds[2];
+    __shared__ int s_flag;
+    __shared__ uint64_t s_match;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+
+    if (!seg_start) {
+        const uint32_t v = blockIdx.x;
+        if (tid < kWave) {
+            const int a = wave_lower_bound(keys, n, v, tile_mask);
+            const int b = v == tile_mask ? n : wave_lower_bound(keys, n, v + 1, tile_mask);
+            if (lane == 0) { s_bounds[0] = a; s_bounds[1] = b; s_flag = 0; }
+        }
+        __syncthreads();
+        const int lo = s_bounds[0], hi = s_bounds[1];
+        const int len = hi - lo;
+        if (len < 2) return;
+        if (len <= min_len) {       // without flags the shorter segments are re-examined here
+            const uint32_t upper = (uint32_t)(keys[lo] >> 32);
+            bool mixed = false;
+            for (int i = tid; i < len; i += kSortBlock) mixed = mixed || (uint32_t)(keys[lo + i] >> 32) != upper;
+            if (mixed) s_flag = 1;
+            __syncthreads();
+            const bool any_mixed = s_flag != 0;
+            __syncthreads();
+            if (!any_mixed) return;
+        }
+        sort_segment_general(keys, values, alt_keys, alt_values, lo, hi, s_cnt, s_wave_sum, &s_flag);
+        return;
+    }
+
+    const uint32_t first_id = blockIdx.x * (uint32_t)kWave;
+    if (tid < kWave) {
+        const uint32_t v = first_id + (uint32_t)lane;
+        bool take = false;
+        if (v < ids) {
+            const int len = seg_start[v + 1] - seg_start[v];
+            take = len > min_len || (len > 1 && ((seg_flags[v >> 5] >> (v & 31)) & 1u));
+        }
+        const uint64_t m = ballot(take);
+        if (lane == 0) s_match = m;
+    }
+    __syncthreads();
+    for (uint64_t todo = s_match; todo; todo &= todo - 1) {
+        const uint32_t v = first_id + (uint32_t)(__ffsll((long long)todo) - 1);
+        sort_segment_general(keys, values, alt_keys, alt_values, seg_start[v], seg_start[v + 1], s_cnt, s_wave_sum, &s_flag);
+    }
+}
+
+constexpr int kCapTiny = 256, kCapSmall = 1024, kCapMedium = 4096, kCapLarge = 8192;
+
 
 } // namespace
 } // namespace fgs
@@ -280,47 +792,86 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
     if (((uintptr_t)gaussian_keys_unsorted | (uintptr_t)gaussian_keys_sorted) % 8 != 0)
         return fail(FGS_E_INVALID, "fgs_sort_gaussian: key buffers must be 8-byte aligned");
 
-    const Workspace ws = workspace_for(num_rendered);
+    const int n = num_rendered;
+    const Workspace ws = workspace_for(n);
     if (sorting_size < ws.total)
         return fail(FGS_E_WORKSPACE, "fgs_sort_gaussian: list_sorting_space holds %zu bytes, %zu needed for %d pairs",
-                    sorting_size, ws.total, num_rendered);
+                    sorting_size, ws.total, n);
 
     const long long tiles_xy = (long long)((width + block_x - 1) / block_x) * ((height + block_y - 1) / block_y);
-    if (tiles_xy > 0xffffffffLL) return fail(FGS_E_INVALID, "fgs_sort_gaussian: too many tiles");
-    const int end_bit = 32 + bit_length((uint32_t)tiles_xy);     // sort.cu:34-39
-    const int passes = (end_bit + 7) / 8;
+    if (tiles_xy >= (1LL << 30)) return fail(FGS_E_INVALID, "fgs_sort_gaussian: too many tiles");
+    const int tile_bits = bit_length((uint32_t)tiles_xy);         // sort.cu:34-39: bits [0, 32 + tile_bits)
+    const uint32_t tile_mask = (1u << tile_bits) - 1u;
+    const int passes = (tile_bits + 7) / 8;
 
     hipStream_t st = (hipStream_t)stream;
     uint64_t* alt_keys = (uint64_t*)(list_sorting_space + ws.alt_keys);
     uint32_t* alt_values = (uint32_t*)(list_sorting_space + ws.alt_values);
-    uint32_t* counters = (uint32_t*)(list_sorting_space + ws.counters);
-    uint32_t* tickets = counters + kMaxPasses * kBins;
-    uint32_t* status = (uint32_t*)(list_sorting_space + ws.status);
+    uint32_t* hist = (uint32_t*)(list_sorting_space + ws.hist);
+    uint32_t* chunk_sums = (uint32_t*)(list_sorting_space + ws.chunk_sums);
 
-    // counters, tickets and the status words of the passes that run are contiguous
-    const size_t zero_words = kCounterWords + (size_t)passes * ws.tiles * kBins;
-    size_t fill_blocks = (zero_words + 2047) / 2048;
-    if (fill_blocks > 2048) fill_blocks = 2048;
-    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)fill_blocks), dim3(256), 0, st, counters, zero_words, 0u);
-
-    const int hist_blocks = ws.tiles < 1024 ? ws.tiles : 1024;
-    hipLaunchKernelGGL(histogram_kernel, dim3(hist_blocks), dim3(kHistBlock), 0, st,
-                       gaussian_keys_unsorted, num_rendered, passes, end_bit, counters);
-    hipLaunchKernelGGL(digit_base_kernel, dim3(passes), dim3(kBins), 0, st, counters);
-
+    // 1. stable partition by tile id, least significant tile digit first
     const uint64_t* src_k = gaussian_keys_unsorted;
     const uint32_t* src_v = gaussian_values_unsorted;
     for (int p = 0; p < passes; p++) {
         const bool to_sorted = ((passes - p) & 1) != 0;      // the last pass lands in the caller's sorted buffers
         uint64_t* dst_k = to_sorted ? gaussian_keys_sorted : alt_keys;
         uint32_t* dst_v = to_sorted ? gaussian_values_sorted : alt_values;
-        const int shift = 8 * p;
-        const int nbits = end_bit - shift < 8 ? end_bit - shift : 8;
-        hipLaunchKernelGGL(reorder_kernel, dim3(ws.tiles), dim3(kSortBlock), 0, st,
-                           src_k, src_v, dst_k, dst_v, num_rendered, shift, nbits,
-                           counters + p * kBins, status + (size_t)p * ws.tiles * kBins, tickets + p);
+        const int shift = 32 + 8 * p;
+        const int nbits = tile_bits - 8 * p < 8 ? tile_bits - 8 * p : 8;
+        hipLaunchKernelGGL(count_kernel, dim3(ws.tiles), dim3(kSortBlock), 0, st, src_k, n, shift, nbits, hist);
+        hipLaunchKernelGGL(chunk_sum_kernel, dim3(ws.chunks), dim3(kBins), 0, st, hist, ws.tiles, ws.chunk, chunk_sums);
+        hipLaunchKernelGGL(offsets_kernel, dim3(ws.chunks), dim3(kBins), 0, st, hist, ws.tiles, ws.chunk, chunk_sums, ws.chunks);
+        hipLaunchKernelGGL(scatter_kernel, dim3(ws.tiles), dim3(kSortBlock), 0, st,
+                           src_k, src_v, dst_k, dst_v, n, shift, nbits, hist);
         src_k = dst_k;
         src_v = dst_v;
     }
-    return check_hip(hipGetLastError(), "radix sort launch");
+
+    // 2. every tile id's segment by depth, in place in the sorted buffers
+    if (n > 1) {
+        const uint32_t ids = 1u << tile_bits;
+        int* seg_start = nullptr;
+        uint32_t* seg_flags = nullptr;
+        if (ids <= kMaxTableIds) {
+            seg_start = (int*)(list_sorting_space + ws.seg_start);
+            seg_flags = (uint32_t*)(list_sorting_space + ws.seg_flags);
+            const unsigned blocks = (unsigned)(((size_t)(n > (int)(ids / 32 + 1) ? n : (int)(ids / 32 + 1)) + 255) / 256);
+            hipLaunchKernelGGL(segment_starts_kernel, dim3(blocks), dim3(256), 0, st,
+                               (const uint64_t*)gaussian_keys_sorted, n, tile_mask, ids, seg_start, seg_flags,
+                               (uint32_t*)(list_sorting_space + ws.seg_lists));
+        }
+        uint64_t* ks = gaussian_keys_sorted;
+        uint32_t* vs = gaussian_values_sorted;
+        uint32_t* seg_counts = (uint32_t*)(list_sorting_space + ws.seg_lists);
+        uint32_t* list_medium = seg_counts + 64;
+        uint32_t* list_large = list_medium + ((size_t)n / 1024 + 2);
+        const uint32_t* no_list = nullptr;
+#define FGS_SEGMENT_CLASS(WAVES, CAP, IDS, MINLEN, GRID, LIST, COUNT)                                         \
+        hipLaunchKernelGGL((segment_sort_kernel<WAVES, CAP, IDS>), dim3(GRID), dim3((WAVES) * kWave), 0, st,  \
+                           ks, vs, n, tile_mask, MINLEN, ids, (const int*)seg_start, seg_flags,               \
+                           (const uint32_t*)(LIST), (const uint32_t*)(COUNT))
+        // one or two tile ids per wave: neighbouring tiles tend to be equally busy, so a wave that
+        // took several of them would become the tail of the launch
+        hipLaunchKernelGGL((segment_sort_wave_kernel<kCapTiny / kWave, 2>), dim3(seg_start ? (ids + 1) / 2 : ids), dim3(kWave),
+                           0, st, ks, vs, n, tile_mask, 1, ids, (const int*)seg_start, seg_flags,
+                           kCapSmall, kCapMedium, kCapLarge, seg_counts, seg_start ? list_medium : nullptr, list_large);
+        if (n > kCapTiny) FGS_SEGMENT_CLASS(1, kCapSmall, 1, kCapTiny, ids, no_list, no_list);
+        if (seg_start) {
+            if (n > kCapSmall) {
+                const unsigned most_m = (unsigned)(n / (kCapSmall + 1) + 1), most_l = (unsigned)(n / (kCapMedium + 1) + 1);
+                FGS_SEGMENT_CLASS(8, kCapMedium, 64, kCapSmall, most_m < 1024u ? most_m : 1024u, list_medium, seg_counts);
+                if (n > kCapMedium)
+                    FGS_SEGMENT_CLASS(16, kCapLarge, 64, kCapMedium, most_l < 256u ? most_l : 256u, list_large, seg_counts + 1);
+            }
+        } else {
+            if (n > kCapSmall) FGS_SEGMENT_CLASS(8, kCapMedium, 64, kCapSmall, ids, no_list, no_list);
+            if (n > kCapMedium) FGS_SEGMENT_CLASS(16, kCapLarge, 64, kCapMedium, ids, no_list, no_list);
+        }
+#undef FGS_SEGMENT_CLASS
+        hipLaunchKernelGGL(segment_sort_general_kernel, dim3(seg_start ? (ids + kWave - 1) / kWave : ids),
+                           dim3(kSortBlock), 0, st, ks, vs, alt_keys, alt_values, n, tile_mask, kCapLarge, ids,
+                           (const int*)seg_start, (const uint32_t*)seg_flags);
+    }
+    return check_hip(hipGetLastError(), "sort launch");
 }

@@ -236,3 +236,60 @@ def test_full_size_configs(oracle, config):
     """The 1080p / 1M and the 4K / 3M configurations end to end against the oracle."""
     sc = scenes.make(config)
     _check_frame(oracle, sc, sc.cameras[0], 1 << 24)
+
+
+def _sort_case(tile, depth_bits, W, H, junk=None, seed=0):
+    import gpu_pipeline as gp
+    rng = np.random.default_rng(seed)
+    n = tile.size
+    keys = (tile.astype(np.uint64) << np.uint64(32)) | depth_bits.astype(np.uint64)
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    end_bit = 32 + int(gx * gy).bit_length()
+    if junk is not None:
+        keys = keys | (junk.astype(np.uint64) << np.uint64(end_bit))
+    vals = rng.permutation(n).astype(np.uint32)
+    ks, vs = gp.sort(n, W, H, gp.dev(keys.view(np.int64)), gp.dev(vals.view(np.int32)))
+    masked = keys & np.uint64((1 << end_bit) - 1)
+    order = np.argsort(masked, kind="stable")
+    assert np.array_equal(gp.u64(ks)[:n], keys[order])
+    assert np.array_equal(gp.u32(vs)[:n], vals[order])
+
+
+@pytest.mark.parametrize("seg", [1500, 3000, 5000, 8000, 8192, 8193, 40000])
+def test_sort_segment_size_classes(seg):
+    """Tiles holding 1500 ... 40000 pairs: every size class of the per-tile depth sort, with many
+    equal depths and with depths that agree in whole bytes (skipped passes)."""
+    rng = np.random.default_rng(seg)
+    W, H = 1920, 1080
+    tile = np.repeat(np.array([5, 6, 4000, 8159], np.uint32), [seg, 7, seg // 2, seg])
+    rng.shuffle(tile)
+    depth = rng.uniform(1.0, 1.9, tile.size).astype(np.float32)      # same exponent: top byte constant
+    depth[::3] = np.float32(1.5)
+    _sort_case(tile, depth.view(np.uint32), W, H, seed=seg)
+
+
+def test_sort_bits_above_the_range_stay_with_their_pair():
+    """Bits above 32 + bit_length(tiles) are outside the sorted range (sort.cu:34-39) but travel
+    with the key; segments whose keys differ there take the general path."""
+    rng = np.random.default_rng(77)
+    W, H = 640, 480                                   # 1200 tiles -> 11 tile bits
+    n = 60000
+    tile = rng.integers(0, 1200, n).astype(np.uint32)
+    tile[:20000] = 17                                 # one long segment
+    depth = rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32)
+    junk = rng.integers(0, 1 << 10, n).astype(np.uint32)
+    junk[30000:] = 0
+    _sort_case(tile, depth, W, H, junk=junk, seed=1)
+
+
+def test_sort_more_tile_ids_than_the_segment_table():
+    """16400 x 16400 pixels = 1 050 625 tiles: 21 tile bits, three partition passes, and segment
+    bounds found by search instead of the table."""
+    rng = np.random.default_rng(78)
+    W = H = 16400
+    n = 300_000
+    tile = rng.integers(0, 1025 * 1025, n).astype(np.uint32)
+    tile[:5000] = 1_050_624
+    tile[5000:9000] = 0
+    depth = rng.uniform(0.2, 90.0, n).astype(np.float32)
+    _sort_case(tile, depth.view(np.uint32), W, H, seed=2)
