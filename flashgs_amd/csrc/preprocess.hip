@@ -238,11 +238,16 @@ __device__ __forceinline__ uint64_t peek(const uint64_t* slot)
     return __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Executed by the first wave of a workgroup with ticket > 0.  Lane l inspects the workgroup
-// `top - l`; the walk ends at the nearest one that has published a prefix.  Returns the sum of
-// the key counts of all workgroups with a smaller ticket.  *failed is set when a predecessor
-// stayed silent for kSpinLimit polls or reported such a failure itself; the wait is bounded so
-// that every wave of the grid exits whatever happens.
+// Executed by the first wave of a workgroup with ticket > 0.  Returns the sum of the key counts
+// of all workgroups with a smaller ticket.  The wave inspects kLookAhead windows of 64
+// predecessors per round trip to memory (lane l of window u looks at workgroup top - 64u - l)
+// and walks them nearest first; the walk ends at the nearest workgroup that has published a
+// prefix.  The chain of prefixes can only advance one round trip at a time, so the number of
+// predecessors covered per round trip is what bounds how fast workgroups can retire.
+// *failed is set when a predecessor stayed silent for kSpinLimit polls or reported such a failure
+// itself; the wait is bounded so that every wave of the grid exits whatever happens.
+constexpr int kLookAhead = 4;
+
 __device__ __forceinline__ uint32_t look_back(const uint64_t* status, int ticket, uint32_t epoch, bool* failed)
 {
     const int lane = lane_id();
@@ -250,32 +255,39 @@ __device__ __forceinline__ uint32_t look_back(const uint64_t* status, int ticket
     unsigned spins = 0;
     int top = ticket - 1;
     for (;;) {
-        const int j = top - lane;
-        uint64_t w = 0;
-        uint32_t state = 0;
-        uint64_t closing = 0;        // lanes holding a prefix (or poison) word
-        for (;;) {
-            state = 0;
-            if (j >= 0) {
-                w = peek(status + j);
-                if ((uint32_t)(w >> 34) == epoch) state = (uint32_t)(w >> 32) & 3u;
-            }
-            const uint64_t pending = ballot(j >= 0 && state == 0);
-            closing = ballot(state >= kStatePrefix);
-            const uint64_t need = closing ? ((closing & (~closing + 1)) << 1) - 1 : ~0ull;
-            if ((pending & need) == 0) break;
-            if (++spins > kSpinLimit) { *failed = true; return sum; }
-            __builtin_amdgcn_s_sleep(2);
-        }
-        const uint64_t first = closing & (~closing + 1);
-        const uint64_t take = closing ? (first << 1) - 1 : ~0ull;
-        if (ballot(state == kStatePoison) & first) *failed = true;
-        uint32_t v = (j >= 0 && ((take >> lane) & 1)) ? (uint32_t)w : 0u;
+        uint64_t w[kLookAhead];
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) v += (uint32_t)__shfl_xor((int)v, o);
-        sum += v;
-        if (closing || top - kWave < 0) return sum;
-        top -= kWave;
+        for (int u = 0; u < kLookAhead; u++) {
+            const int j = top - u * kWave - lane;
+            w[u] = j >= 0 ? peek(status + j) : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < kLookAhead; u++) {
+            const int j = top - u * kWave - lane;
+            uint64_t word = w[u];
+            uint32_t state;
+            uint64_t closing;        // lanes holding a prefix (or poison) word
+            for (;;) {
+                state = 0;
+                if (j >= 0 && (uint32_t)(word >> 34) == epoch) state = (uint32_t)(word >> 32) & 3u;
+                const uint64_t pending = ballot(j >= 0 && state == 0);
+                closing = ballot(state >= kStatePrefix);
+                const uint64_t need = closing ? ((closing & (~closing + 1)) << 1) - 1 : ~0ull;
+                if ((pending & need) == 0) break;
+                if (++spins > kSpinLimit) { *failed = true; return sum; }
+                __builtin_amdgcn_s_sleep(2);
+                if (j >= 0) word = peek(status + j);
+            }
+            const uint64_t first = closing & (~closing + 1);
+            const uint64_t take = closing ? (first << 1) - 1 : ~0ull;
+            if (ballot(state == kStatePoison) & first) *failed = true;
+            uint32_t v = (j >= 0 && ((take >> lane) & 1)) ? (uint32_t)word : 0u;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += (uint32_t)__shfl_xor((int)v, o);
+            sum += v;
+            if (closing || top - (u + 1) * kWave < 0) return sum;
+        }
+        top -= kLookAhead * kWave;
     }
 }
 

@@ -5,7 +5,7 @@
 //
 // Blend layout: one wave64 owns one tile.  A tile is made of 16x16-pixel sub-tiles (1 for 16x16,
 // 2 for 32x16, 4 for 32x32); lane l shades the 2x2 pixel quad at (2*(l%8), 2*(l/8)) of every
-// sub-tile, so the quadratic form is evaluated with shared column/row terms.  Gaussians are
+// sub-tile; the quadratic form is evaluated at one pixel of the quad and stepped to the others.  Gaussians are
 // staged 64 at a time into LDS (one per lane: index -> centre, conic+opacity, colour) while the
 // loads of the following batch are already in flight, and the wave walks the batch reading LDS
 // at wave-uniform addresses.  After every second Gaussian one ballot tests whether all pixels of
@@ -54,8 +54,11 @@ __device__ __forceinline__ uint8_t encode_u8(float x)
 }
 
 // One Gaussian applied to this lane's 2x2 pixel quad (render.cu:40-52 for each pixel).  The
-// quadratic is split into a column part A[i], a row part B[j] and the cross term, so the four
-// evaluations share most of the arithmetic.
+// exponent q(dx, dy) = w + cx dx^2 + cz dy^2 + cy dx dy is evaluated once, at the quad's first
+// pixel, and stepped to its neighbours with the exact differences of the quadratic
+// (q(dx-1, dy) - q(dx, dy) = cx - 2 cx dx - cy dy, and likewise in y; the mixed step adds cy).
+// dx, dy are offsets from the Gaussian's own centre, so every term has the magnitude of the
+// exponent itself and the stepping loses nothing that matters against the 2e-3 image tolerance.
 struct Quad {
     float T[2][2], r[2][2], g[2][2], b[2][2];
 };
@@ -63,16 +66,15 @@ struct Quad {
 __device__ __forceinline__ void shade_quad(Quad& q, float px0, float py0, const float4 a, const float4 b4, const float blue)
 {
     // a = (centre x, centre y, conic x, conic y), b4 = (conic z, log2 opacity, red, green)
-    const float dx0 = a.x - px0, dx1 = a.x - (px0 + 1.0f);
-    const float dy0 = a.y - py0, dy1 = a.y - (py0 + 1.0f);
-    const float A0 = a.z * dx0 * dx0, A1 = a.z * dx1 * dx1;
-    const float B0 = b4.y + b4.x * dy0 * dy0, B1 = b4.y + b4.x * dy1 * dy1;
-    const float E0 = a.w * dx0, E1 = a.w * dx1;
+    const float dx = a.x - px0, dy = a.y - py0;
+    const float tx = a.z * dx, ty = b4.x * dy, txy = a.w * dx;
     float pw[2][2];
-    pw[0][0] = (A0 + B0) + E0 * dy0;
-    pw[0][1] = (A1 + B0) + E1 * dy0;
-    pw[1][0] = (A0 + B1) + E0 * dy1;
-    pw[1][1] = (A1 + B1) + E1 * dy1;
+    pw[0][0] = b4.y + tx * dx + ty * dy + txy * dy;
+    const float step_x = (a.z - 2.0f * tx) - a.w * dy;          // to the pixel at x + 1
+    const float step_y = (b4.x - 2.0f * ty) - txy;             // to the pixel at y + 1
+    pw[0][1] = pw[0][0] + step_x;
+    pw[1][0] = pw[0][0] + step_y;
+    pw[1][1] = (pw[0][1] + step_y) + a.w;
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
