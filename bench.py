@@ -28,8 +28,11 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3         # MI355X fp32 vector, published (packed FMA)
 LANE_SLOTS_PER_S = 256 * 4 * 16 * 2.4e9   # VALU issue slots per second without packed math
+# HBM bytes per blend launch on the headline configuration, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE scaled by the readings of a 256 MiB copy (profiles/frame_cfg2_4K_hbm_traffic.txt); other workloads: not measured
+BLEND_TRAFFIC_BYTES = {"cfg2_3M_4K": 1416360878}
 FLOP_PER_EVAL = 19               # render.cu:40-52: 2 sub, 6 mul + 3 add, 1 mul, 3 FMA, 1 sub
-SLOTS_PER_EVAL = 17              # 13 VALU with FMA contraction + a quarter-rate exp2
+SLOTS_PER_EVAL = 17              # 13 VALU with FMA contraction + a quarter-rate exp2 (the reference formulation)
 
 
 def parse():
@@ -40,6 +43,8 @@ def parse():
     ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (default: the 4K / 3M headline)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-reps", type=int, default=3)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 256 MiB device-to-device copy, as the known-size reference for FETCH_SIZE / WRITE_SIZE")
     return ap.parse_args()
 
 
@@ -146,6 +151,12 @@ def main():
     for i in range(args.warmup):
         frame(cams[i % len(cams)])
     torch.cuda.synchronize()
+    if args.copy_calibration:
+        src = torch.ones(64 << 20, device=dev, dtype=torch.float32)      # 256 MiB read + 256 MiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     events = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(args.steps)]
     frame_ms, Ks = [], []
@@ -185,12 +196,15 @@ def main():
     else:
         stages["preprocess"] = dict(ms=round(stage_ms["preprocess"], 4), bound="hbm")
     hbm("sort", K * (8 + 24 * passes))
+    tile_passes = (int(tiles).bit_length() + 7) // 8
+    stages["sort"]["design_bytes"] = int(K * (32 * tile_passes + 8 + 24))   # count + scatter per tile digit, starts, segment sort
     hbm("ranges", 8 * K + 16 * tiles)
     stages["readback"] = dict(ms=round(stage_ms["readback"], 4), bound="host latency (4-byte read + sync)")
 
     blend_ms = stage_ms["blend"]
-    roofline = dict(kernel="blend_kernel<1,1> (16x16 tile, 4 wave64)", bound="valu", achieved=None,
-                    peak=FP32_PEAK_TFLOPS, unit="TFLOP/s", frac=None, traffic=None, launch_ms=round(blend_ms, 4))
+    roofline = dict(kernel="blend_kernel<1,1> (16x16 tile, one wave64, 2x2 pixels per lane)", bound="valu", achieved=None,
+                    peak=FP32_PEAK_TFLOPS, unit="TFLOP/s", frac=None, traffic=BLEND_TRAFFIC_BYTES.get(sc.name),
+                    launch_ms=round(blend_ms, 4))
     if walked is not None and len(cams) == 1:
         evals = 256 * walked
         tflops = FLOP_PER_EVAL * evals / (blend_ms * 1e-3) / 1e12

@@ -56,4 +56,20 @@ __device__ __forceinline__ float bcast_f(float v, int src_lane)
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src_lane));
 }
 
+// Inclusive prefix sum over the 64 lanes of a wave with data-parallel-primitive moves (VALU only):
+// shifts by 1, 2, 4, 8 inside each row of 16 lanes, then the last lane of rows 0 and 2 is added
+// to rows 1 and 3, then lane 31 to rows 2 and 3.  Lanes without a source add 0.
+__device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t x)
+{
+    constexpr int kRowShr1 = 0x111, kRowShr2 = 0x112, kRowShr4 = 0x114, kRowShr8 = 0x118;
+    constexpr int kRowBcast15 = 0x142, kRowBcast31 = 0x143;
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, kRowShr1, 0xf, 0xf, false);
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, kRowShr2, 0xf, 0xf, false);
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, kRowShr4, 0xf, 0xf, false);
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, kRowShr8, 0xf, 0xf, false);
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, kRowBcast15, 0xa, 0xf, false);
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, kRowBcast31, 0xc, 0xf, false);
+    return x;
+}
+
 } // namespace fgs

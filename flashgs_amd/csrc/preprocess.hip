@@ -401,12 +401,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     // stashes at most kStashCap candidates; what does not fit, and every larger rectangle, is
     // tested by the whole wave, 64 tiles a step, once to count and once more to emit.
     const bool flat_ok = has_tiles && area <= kWave && pack_ok;
-    uint32_t cand_incl = flat_ok ? (uint32_t)area : 0u;
-#pragma unroll
-    for (int o = 1; o < kWave; o <<= 1) {
-        uint32_t up = (uint32_t)__shfl_up((int)cand_incl, o);
-        if (lane >= o) cand_incl += up;
-    }
+    uint32_t cand_incl = wave_inclusive_sum(flat_ok ? (uint32_t)area : 0u);
     const bool flat = flat_ok && cand_incl <= (uint32_t)kStashCap;
     const bool large = has_tiles && !flat;
     // lanes that drop out are at the end of the scan order, so the prefix of the others is unchanged
@@ -477,12 +472,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     }
 
     // ---- slots: wave scan, block scan, chained scan over workgroups ----
-    uint32_t incl = count;
-#pragma unroll
-    for (int o = 1; o < kWave; o <<= 1) {
-        uint32_t up = (uint32_t)__shfl_up((int)incl, o);
-        if (lane >= o) incl += up;
-    }
+    uint32_t incl = wave_inclusive_sum(count);
     const uint32_t wave_total = (uint32_t)bcast_i((int)incl, kWave - 1);
     if (lane == 0) s_wave_total[wave] = wave_total;
     __syncthreads();
@@ -531,12 +521,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     const uint32_t depth_bits = __float_as_uint(depth);
     {
         // stash entry e of owner o goes to slot(o) + (e - entries before o's first)
-        uint32_t before = flat_count;
-#pragma unroll
-        for (int o = 1; o < kWave; o <<= 1) {
-            uint32_t up = (uint32_t)__shfl_up((int)before, o);
-            if (lane >= o) before += up;
-        }
+        uint32_t before = wave_inclusive_sum(flat_count);
         const uint32_t delta = my_slot - (before - flat_count);
         const uint32_t gidx_base = (uint32_t)(ticket * kBlock + wave * kWave);
         for (int e0 = 0; e0 < n_stash; e0 += kWave) {

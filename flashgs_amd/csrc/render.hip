@@ -92,7 +92,7 @@ template <int SX, int SY>
 __global__ __launch_bounds__(kWave) void blend_kernel(
     const int2* __restrict__ ranges,
     const uint32_t* __restrict__ point_list,
-    int width, int height, int tiles_x,
+    int width, int height, int tiles_x, int tiles_y,
     const float2* __restrict__ points_xy,
     const float4* __restrict__ rgb_depth,
     const float4* __restrict__ conic_opacity,
@@ -106,7 +106,18 @@ __global__ __launch_bounds__(kWave) void blend_kernel(
     __shared__ float s_c[kWave];               // blue
 
     const int lane = threadIdx.x;
-    const int tile_x = blockIdx.x, tile_y = blockIdx.y;
+    // Workgroup -> tile.  The hardware deals consecutive workgroups out to the 8 XCDs in turn, and
+    // every XCD has its own L2.  Neighbouring tiles share most of their Gaussians, so each XCD is
+    // given whole 8x8 blocks of tiles (its workgroups g = 8*slot + xcd walk blocks xcd, xcd+8, ...
+    // 64 tiles at a time): a Gaussian's attribute lines are then fetched into one L2 once instead
+    // of into several L2s once per tile.
+    const int group = blockIdx.x;
+    const int xcd = group & 7, slot = group >> 3;
+    const int blocks_x = (tiles_x + 7) >> 3;
+    const int block = (slot >> 6) * 8 + xcd, inner = slot & 63;
+    const int tile_x = (block % blocks_x) * 8 + (inner & 7);
+    const int tile_y = (block / blocks_x) * 8 + (inner >> 3);
+    if (tile_x >= tiles_x || tile_y >= tiles_y) return;
     const int2 range = ranges[tile_y * tiles_x + tile_x];
     const int n = range.y - range.x;
 
@@ -250,10 +261,14 @@ int blend_impl(int block_x, int block_y, int width, int height,
         return fail(FGS_E_INVALID, "%s: rgb_depth/conic_opacity must be 16-byte aligned, points_xy/ranges 8-byte aligned", who);
     const int tiles_x = (width + block_x - 1) / block_x, tiles_y = (height + block_y - 1) / block_y;
     hipStream_t st = (hipStream_t)stream;
-    const dim3 grid(tiles_x, tiles_y);
+    // one workgroup per tile of the image padded to whole 8x8 blocks of tiles, blocks padded to a multiple of 8
+    const long long blocks = (long long)((tiles_x + 7) / 8) * ((tiles_y + 7) / 8);
+    const long long groups = (blocks + 7) / 8 * 8 * 64;
+    if (groups > 0x7fffffffLL) return fail(FGS_E_INVALID, "%s: image too large", who);
+    const dim3 grid((unsigned)groups);
 #define FGS_LAUNCH_BLEND(SX, SY)                                                                        \
     hipLaunchKernelGGL((blend_kernel<SX, SY>), grid, dim3(kWave), 0, st,                                \
-                       (const int2*)ranges, values_sorted, width, height, tiles_x,                      \
+                       (const int2*)ranges, values_sorted, width, height, tiles_x, tiles_y,             \
                        (const float2*)points_xy, (const float4*)rgb_depth, (const float4*)conic_opacity, \
                        bg[0], bg[1], bg[2], out_u8, out_f32)
     if (sx == 1 && sy == 1) FGS_LAUNCH_BLEND(1, 1);

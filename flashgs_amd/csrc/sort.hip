@@ -120,12 +120,7 @@ __global__ __launch_bounds__(kBins) void offsets_kernel(uint32_t* __restrict__ h
         }
     }
     // exclusive scan of the digit totals over the 256 digits
-    uint32_t incl = total;
-#pragma unroll
-    for (int o = 1; o < kWave; o <<= 1) {
-        uint32_t up = (uint32_t)__shfl_up((int)incl, o);
-        if (lane >= o) incl += up;
-    }
+    uint32_t incl = wave_inclusive_sum(total);
     if (lane == kWave - 1) s_wave[wave] = incl;
     __syncthreads();
     uint32_t digit_base = incl - total;
@@ -223,12 +218,7 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
         s_count[w][d] = total;
         total += c;
     }
-    uint32_t incl = total;
-#pragma unroll
-    for (int o = 1; o < kWave; o <<= 1) {
-        uint32_t up = (uint32_t)__shfl_up((int)incl, o);
-        if (lane >= o) incl += up;
-    }
+    uint32_t incl = wave_inclusive_sum(total);
     if (lane == kWave - 1) s_wave_sum[wave] = incl;
     __syncthreads();
     uint32_t before_wave = 0;
@@ -337,12 +327,7 @@ __device__ __forceinline__ bool counting_pass(const KeyT* src_k, const uint32_t*
         for (int q = 0; q < 4; q++) {
             const uint32_t c = cnt[0][q * kWave + lane];
             any_full = any_full || c == (uint32_t)n;
-            uint32_t incl = c;
-#pragma unroll
-            for (int o = 1; o < kWave; o <<= 1) {
-                uint32_t up = (uint32_t)__shfl_up((int)incl, o);
-                if (lane >= o) incl += up;
-            }
+            uint32_t incl = wave_inclusive_sum(c);
             cnt[0][q * kWave + lane] = base + incl - c;
             base += (uint32_t)bcast_i((int)incl, kWave - 1);
         }
@@ -358,12 +343,7 @@ __device__ __forceinline__ bool counting_pass(const KeyT* src_k, const uint32_t*
                 total += c;
             }
             if (total == (uint32_t)n) *flag = 1;
-            uint32_t incl = total;
-#pragma unroll
-            for (int o = 1; o < kWave; o <<= 1) {
-                uint32_t up = (uint32_t)__shfl_up((int)incl, o);
-                if (lane >= o) incl += up;
-            }
+            uint32_t incl = wave_inclusive_sum(total);
             if (lane == kWave - 1) wave_sum[wave] = incl;
             total = incl - total;             // exclusive inside this wave's 64 digits
         }
@@ -576,12 +556,7 @@ __device__ __forceinline__ void sort_segment_wave(uint64_t* __restrict__ keys, u
         for (int q = 0; q < 4; q++) {
             const uint32_t c = cnt[q * kWave + lane];
             any_full = any_full || c == (uint32_t)len;
-            uint32_t incl = c;
-#pragma unroll
-            for (int o = 1; o < kWave; o <<= 1) {
-                uint32_t up = (uint32_t)__shfl_up((int)incl, o);
-                if (lane >= o) incl += up;
-            }
+            uint32_t incl = wave_inclusive_sum(c);
             cnt[q * kWave + lane] = base + incl - c;
             base += (uint32_t)bcast_i((int)incl, kWave - 1);
         }
