@@ -19,7 +19,6 @@
 #include "fgs_internal.h"
 
 #include <mutex>
-#include <stdlib.h>
 
 namespace fgs {
 namespace {
@@ -307,8 +306,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     int64_t capacity,            // <= 0: unchecked
     uint64_t* __restrict__ status,
     uint32_t epoch,
-    int num_blocks,
-    int exp_flags)
+    int num_blocks)
 {
     __shared__ uint32_t s_wave_total[kWavesPerBlock];
     __shared__ uint32_t s_block_base;
@@ -496,7 +494,6 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         reinterpret_cast<float4*>(conic_opacity)[idx] =
             make_float4((-0.5f * log2e) * conx, -log2e * cony, (-0.5f * log2e) * conz, log2_op);
         float rgb[3];
-        if (exp_flags & 8) { rgb[0] = rgb[1] = rgb[2] = 0.5f; } else
         sh_to_rgb(shs + 48 * (size_t)idx, px, py, pz, cam, rgb);
         reinterpret_cast<float4*>(rgb_depth)[idx] = make_float4(rgb[0], rgb[1], rgb[2], depth);
     }
@@ -505,7 +502,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         bool timed_out = false;
         uint32_t excl;
         if (ticket == 0) excl = (uint32_t)*curr_offset;     // the caller's starting offset (example.py:69 zeroes it)
-        else excl = (exp_flags & 4) ? 0u : look_back(status, ticket, epoch, &timed_out);
+        else excl = look_back(status, ticket, epoch, &timed_out);
         if (lane == 0) {
             publish(status + ticket, pack_status(epoch, timed_out ? kStatePoison : kStatePrefix, excl + block_total));
             s_block_base = excl;
@@ -712,6 +709,6 @@ extern "C" int fgs_preprocess(int P,
     hipLaunchKernelGGL(preprocess_kernel, dim3(num_blocks), dim3(kBlock), 0, st,
                        P, positions, shs, opacities, cov3Ds, cam, points_xy, rgb_depth, conic_opacity,
                        gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset, key_capacity,
-                       s->status, s->epoch, num_blocks, getenv("FGS_EXP") ? atoi(getenv("FGS_EXP")) : 0);
+                       s->status, s->epoch, num_blocks);
     return check_hip(hipGetLastError(), "preprocess_kernel launch");
 }
