@@ -831,7 +831,7 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         hipLaunchKernelGGL((segment_sort_wave_kernel<kCapTiny / kWave, 2>), dim3(seg_start ? (ids + 1) / 2 : ids), dim3(kWave),
                            0, st, ks, vs, n, tile_mask, 1, ids, (const int*)seg_start, seg_flags,
                            kCapSmall, kCapMedium, kCapLarge, seg_counts, seg_start ? list_medium : nullptr, list_large);
-        if (n > kCapTiny) FGS_SEGMENT_CLASS(1, kCapSmall, 1, kCapTiny, ids, no_list, no_list);
+        if (n > kCapTiny) FGS_SEGMENT_CLASS(4, kCapSmall, 1, kCapTiny, ids, no_list, no_list);
         if (seg_start) {
             if (n > kCapSmall) {
                 const unsigned most_m = (unsigned)(n / (kCapSmall + 1) + 1), most_l = (unsigned)(n / (kCapMedium + 1) + 1);
