@@ -26,6 +26,8 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kStashCap = 1024;         // flat candidates (and so stashed hits) per wave
+constexpr int kHugeMin = 1024;          // rectangles with more tiles than this are tested by the whole workgroup
+constexpr int kHugeCap = 16;            // such rectangles per workgroup; further ones stay with their wave
 constexpr unsigned kSpinLimit = 1u << 22;   // polls before a chained-scan wait gives up
 
 struct Camera {
@@ -162,6 +164,17 @@ __device__ __forceinline__ bool tile_hit(int x, int y, int bx, int by, float cx,
     b = -2.0f * cony * dy;
     c = conz * dy * dy - w;
     return segment_hits(a, b, c, cx, fminx, fmaxx);
+}
+
+// j / w and j % w for 0 <= j, 1 <= w.  Below 2^20 the quotient comes from a reciprocal estimate
+// (off by less than 1/4 there) corrected by one step either way.
+__device__ __forceinline__ void div_mod(int j, int w, int& q, int& r)
+{
+    if (j >= (1 << 20)) { q = j / w; r = j - q * w; return; }
+    q = (int)(((float)j + 0.5f) * __builtin_amdgcn_rcpf((float)w));
+    r = j - q * w;
+    if (r < 0) { q--; r += w; }
+    else if (r >= w) { q++; r -= w; }
 }
 
 // preprocess.cu:13-34, :145-185
@@ -313,10 +326,18 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     __shared__ uint32_t s_stash[kWavesPerBlock][kStashCap];     // hits of the flat candidates, in emission order
     __shared__ uint64_t s_hits[kWavesPerBlock][kStashCap / kWave + 1];
     __shared__ uint8_t s_owner[kWavesPerBlock][kStashCap];      // flat candidate -> lane that owns it
+    // rectangles too big for one wave: parameters, per-wave hit counts, first key slot
+    __shared__ float s_huge_f[kHugeCap][6];
+    __shared__ int s_huge_i[kHugeCap][4];
+    __shared__ uint32_t s_huge_u[kHugeCap][3];                  // depth bits, Gaussian index, first slot
+    __shared__ uint32_t s_huge_cnt[kHugeCap][kWavesPerBlock];
+    __shared__ int s_nhuge;
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
+    if (tid == 0) s_nhuge = 0;
+    __syncthreads();
 
     // Workgroups are numbered by their index: the hardware dispatches them in index order, so
     // every workgroup with a smaller index is already running or finished when this one waits
@@ -401,7 +422,21 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     const bool flat_ok = has_tiles && area <= kWave && pack_ok;
     uint32_t cand_incl = wave_inclusive_sum(flat_ok ? (uint32_t)area : 0u);
     const bool flat = flat_ok && cand_incl <= (uint32_t)kStashCap;
-    const bool large = has_tiles && !flat;
+    // A rectangle of thousands of tiles would keep one wave busy for a long time while every later
+    // workgroup waits for this workgroup's count: such rectangles are put on a list and all waves
+    // of the workgroup share the testing, a contiguous quarter of the tiles each.
+    int huge_slot = -1;
+    if (has_tiles && area > kHugeMin && area < (1 << 26)) {
+        const int e = atomicAdd(&s_nhuge, 1);
+        if (e < kHugeCap) {
+            huge_slot = e;
+            s_huge_f[e][0] = cx; s_huge_f[e][1] = cy; s_huge_f[e][2] = conx;
+            s_huge_f[e][3] = cony; s_huge_f[e][4] = conz; s_huge_f[e][5] = power;
+            s_huge_i[e][0] = rminx; s_huge_i[e][1] = rminy; s_huge_i[e][2] = rw; s_huge_i[e][3] = area;
+            s_huge_u[e][0] = __float_as_uint(depth); s_huge_u[e][1] = (uint32_t)idx;
+        }
+    }
+    const bool large = has_tiles && !flat && huge_slot < 0;
     // lanes that drop out are at the end of the scan order, so the prefix of the others is unchanged
     const uint32_t cand_excl = cand_incl - (uint32_t)area;
     const uint64_t flat_lanes = ballot(flat);
@@ -461,12 +496,43 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
             const int j = base + lane;
             bool ok = false;
             if (j < garea) {
-                const int ty = j / grw, tx = j - ty * grw;
+                int tx, ty;
+                div_mod(j, grw, ty, tx);
                 ok = tile_hit(gminx + tx, gminy + ty, cam.bx, cam.by, gcx, gcy, gconx, gcony, gconz, gpower);
             }
             total += (uint32_t)__popcll(ballot(ok));
         }
         if (lane == src) count = total;
+    }
+
+    // the listed rectangles: wave w counts tiles [w*part, (w+1)*part) of each
+    __syncthreads();
+    const int n_huge = min(s_nhuge, kHugeCap);
+    for (int e = 0; e < n_huge; e++) {
+        const float gcx = s_huge_f[e][0], gcy = s_huge_f[e][1];
+        const float gconx = s_huge_f[e][2], gcony = s_huge_f[e][3], gconz = s_huge_f[e][4], gpower = s_huge_f[e][5];
+        const int gminx = s_huge_i[e][0], gminy = s_huge_i[e][1], grw = s_huge_i[e][2], garea = s_huge_i[e][3];
+        const int part = ((garea + kWavesPerBlock - 1) / kWavesPerBlock + kWave - 1) / kWave * kWave;
+        const int j_lo = min(garea, wave * part), j_hi = min(garea, j_lo + part);
+        uint32_t total = 0;
+        for (int base = j_lo; base < j_hi; base += kWave) {
+            const int j = base + lane;
+            bool ok = false;
+            if (j < j_hi) {
+                int tx, ty;
+                div_mod(j, grw, ty, tx);
+                ok = tile_hit(gminx + tx, gminy + ty, cam.bx, cam.by, gcx, gcy, gconx, gcony, gconz, gpower);
+            }
+            total += (uint32_t)__popcll(ballot(ok));
+        }
+        if (lane == 0) s_huge_cnt[e][wave] = total;
+    }
+    if (n_huge > 0) {
+        __syncthreads();
+        if (huge_slot >= 0) {
+            count = 0;
+            for (int w = 0; w < kWavesPerBlock; w++) count += s_huge_cnt[huge_slot][w];
+        }
     }
 
     // ---- slots: wave scan, block scan, chained scan over workgroups ----
@@ -516,6 +582,39 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     // ---- emit ----
     const uint64_t cap = capacity > 0 ? (uint64_t)capacity : ~0ull;
     const uint32_t depth_bits = __float_as_uint(depth);
+    if (n_huge > 0) {
+        if (huge_slot >= 0) s_huge_u[huge_slot][2] = my_slot;
+        __syncthreads();
+        for (int e = 0; e < n_huge; e++) {
+            const float gcx = s_huge_f[e][0], gcy = s_huge_f[e][1];
+            const float gconx = s_huge_f[e][2], gcony = s_huge_f[e][3], gconz = s_huge_f[e][4], gpower = s_huge_f[e][5];
+            const int gminx = s_huge_i[e][0], gminy = s_huge_i[e][1], grw = s_huge_i[e][2], garea = s_huge_i[e][3];
+            const uint32_t gdepth = s_huge_u[e][0], gidx = s_huge_u[e][1];
+            uint64_t slot = s_huge_u[e][2];
+            for (int w = 0; w < wave; w++) slot += s_huge_cnt[e][w];
+            if (s_huge_cnt[e][wave] == 0) continue;
+            const int part = ((garea + kWavesPerBlock - 1) / kWavesPerBlock + kWave - 1) / kWave * kWave;
+            const int j_lo = min(garea, wave * part), j_hi = min(garea, j_lo + part);
+            for (int base = j_lo; base < j_hi; base += kWave) {
+                const int j = base + lane;
+                bool ok = false;
+                int tx = 0, ty = 0;
+                if (j < j_hi) {
+                    div_mod(j, grw, ty, tx);
+                    ok = tile_hit(gminx + tx, gminy + ty, cam.bx, cam.by, gcx, gcy, gconx, gcony, gconz, gpower);
+                }
+                const uint64_t hits = ballot(ok);
+                if (ok) {
+                    const uint64_t dst = slot + (uint64_t)popc_below(hits);
+                    if (dst < cap) {
+                        keys[dst] = ((uint64_t)(uint32_t)((gminy + ty) * cam.gx + gminx + tx) << 32) | gdepth;
+                        values[dst] = gidx;
+                    }
+                }
+                slot += (uint64_t)__popcll(hits);
+            }
+        }
+    }
     {
         // stash entry e of owner o goes to slot(o) + (e - entries before o's first)
         uint32_t before = wave_inclusive_sum(flat_count);
@@ -551,7 +650,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
             bool ok = false;
             int tx = 0, ty = 0;
             if (j < garea) {
-                ty = j / grw; tx = j - ty * grw;
+                div_mod(j, grw, ty, tx);
                 ok = tile_hit(gminx + tx, gminy + ty, cam.bx, cam.by, gcx, gcy, gconx, gcony, gconz, gpower);
             }
             const uint64_t hits = ballot(ok);
