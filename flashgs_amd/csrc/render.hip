@@ -53,37 +53,55 @@ __device__ __forceinline__ uint8_t encode_u8(float x)
     return (uint8_t)v;
 }
 
-// One Gaussian applied to this lane's 2x2 pixel quad (render.cu:40-52 for each pixel).  The
-// exponent q(dx, dy) = w + cx dx^2 + cz dy^2 + cy dx dy is evaluated once, at the quad's first
-// pixel, and stepped to its neighbours with the exact differences of the quadratic
-// (q(dx-1, dy) - q(dx, dy) = cx - 2 cx dx - cy dy, and likewise in y; the mixed step adds cy).
-// dx, dy are offsets from the Gaussian's own centre, so every term has the magnitude of the
-// exponent itself and the stepping loses nothing that matters against the 2e-3 image tolerance.
+// The exponent of a Gaussian at a pixel, q = w + cx dx^2 + cz dy^2 + cy dx dy with (dx, dy) the
+// offset of the pixel from the Gaussian's centre (render.cu:42-45), is split over the tile's own
+// pixel grid.  With (X, Y) the pixel's integer offset from the tile centre and (ex, ey) the
+// Gaussian centre's offset from the tile centre, dx = ex - X, dy = ey - Y and
+//     q = F(X) + G(Y) + cy X Y,
+//     F(X) = (w - cy ex ey) + dx (cx dx + cy ey),      G(Y) = dy (cz dy + cy ex).
+// F and G depend on one coordinate only: for every staged Gaussian they are tabulated once per
+// tile column and row (kFx + kGy values) by the staging lanes, and a lane gets the exponents of
+// its 2x2 quad from two table reads, four additions and four FMAs with its own constants X*Y.
+// All terms are of the magnitude of the exponent itself or of cy*|X|*|Y| with |X|, |Y| <= 16, so
+// nothing is lost against the 2e-3 image tolerance.
 struct Quad {
     float T[2][2], r[2][2], g[2][2], b[2][2];
 };
 
-__device__ __forceinline__ void shade_quad(Quad& q, float px0, float py0, const float4 a, const float4 b4, const float blue)
+constexpr int kBatch = 32;        // Gaussians staged per round: lanes 0-31 tabulate F, lanes 32-63 G
+
+// A read that stays where it is written: the compiler neither sinks it to its first use nor drops
+// it when the value turns out unused (volatile on the vector type keeps it one wide LDS read).
+template <typename V>
+__device__ __forceinline__ V lds_read(const char* p)
 {
-    // a = (centre x, centre y, conic x, conic y), b4 = (conic z, log2 opacity, red, green)
-    const float dx = a.x - px0, dy = a.y - py0;
-    const float tx = a.z * dx, ty = b4.x * dy, txy = a.w * dx;
-    float pw[2][2];
-    pw[0][0] = b4.y + tx * dx + ty * dy + txy * dy;
-    const float step_x = (a.z - 2.0f * tx) - a.w * dy;          // to the pixel at x + 1
-    const float step_y = (b4.x - 2.0f * ty) - txy;             // to the pixel at y + 1
-    pw[0][1] = pw[0][0] + step_x;
-    pw[1][0] = pw[0][0] + step_y;
-    pw[1][1] = (pw[0][1] + step_y) + a.w;
+    typedef float Native __attribute__((ext_vector_type(sizeof(V) / sizeof(float))));
+    const Native n = *(const volatile __attribute__((address_space(3))) Native*)p;
+    V v;
+    __builtin_memcpy(&v, &n, sizeof(V));
+    return v;
+}
+
+// what a lane reads of one staged Gaussian: (cy, red, green, blue), F at its columns, G at its rows
+template <int SX, int SY>
+struct StagedT {
+    float4 u;
+    float2 f[SX], g[SY];
+};
+
+__device__ __forceinline__ void shade_quad(Quad& q, const float xy[2][2], const float2 f, const float2 g, const float4 u)
+{
+    // u = (cy, red, green, blue)
+    const float fx[2] = {f.x, f.y}, gy[2] = {g.x, g.y};
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            const float alpha = __builtin_amdgcn_exp2f(pw[j][i]);
+            const float alpha = __builtin_amdgcn_exp2f(__builtin_fmaf(u.x, xy[j][i], fx[i] + gy[j]));
             const float at = alpha * q.T[j][i];
-            q.r[j][i] += b4.z * at;
-            q.g[j][i] += b4.w * at;
-            q.b[j][i] += blue * at;
+            q.r[j][i] += u.y * at;
+            q.g[j][i] += u.z * at;
+            q.b[j][i] += u.w * at;
             q.T[j][i] -= at;
         }
 }
@@ -100,10 +118,12 @@ __global__ __launch_bounds__(kWave) void blend_kernel(
     uint8_t* __restrict__ out_u8,
     float* __restrict__ out_f32)
 {
+    using Staged = StagedT<SX, SY>;
     constexpr int kSub = SX * SY;              // 16x16 sub-tiles per tile = quads per lane
-    __shared__ float4 s_a[kWave];              // centre x, centre y, conic x, conic y
-    __shared__ float4 s_b[kWave];              // conic z, log2 opacity, red, green
-    __shared__ float s_c[kWave];               // blue
+    constexpr int kFx = 16 * SX, kGy = 16 * SY;
+    constexpr int kTab = kFx > kGy ? kFx : kGy;
+    constexpr int kRec = kFx + kGy + 4;        // floats per staged Gaussian: F table, G table, (cy, r, g, b)
+    __shared__ __align__(16) float s_rec[kBatch * kRec];
 
     const int lane = threadIdx.x;
     // Workgroup -> tile.  The hardware deals consecutive workgroups out to the 8 XCDs in turn, and
@@ -123,65 +143,120 @@ __global__ __launch_bounds__(kWave) void blend_kernel(
 
     // lane -> 2x2 quad of every 16x16 sub-tile
     const int qx = (lane & 7) * 2, qy = (lane >> 3) * 2;
+    const float centre_x = (float)(tile_x * kFx + kFx / 2), centre_y = (float)(tile_y * kGy + kGy / 2);
     int pix_x[kSub], pix_y[kSub];
-    float pxf[kSub], pyf[kSub];
+    float xy[kSub][2][2];                      // X*Y of the quad's pixels, offsets from the tile centre
     Quad quad[kSub];
 #pragma unroll
     for (int s = 0; s < kSub; s++) {
-        pix_x[s] = tile_x * (16 * SX) + (s % SX) * 16 + qx;
-        pix_y[s] = tile_y * (16 * SY) + (s / SX) * 16 + qy;
-        pxf[s] = (float)pix_x[s];
-        pyf[s] = (float)pix_y[s];
+        const int lx = (s % SX) * 16 + qx, ly = (s / SX) * 16 + qy;
+        pix_x[s] = tile_x * kFx + lx;
+        pix_y[s] = tile_y * kGy + ly;
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int i = 0; i < 2; i++) {
+                xy[s][j][i] = (float)((lx + i - kFx / 2) * (ly + j - kGy / 2));
                 quad[s].T[j][i] = 1.0f;
                 quad[s].r[j][i] = 0.0f; quad[s].g[j][i] = 0.0f; quad[s].b[j][i] = 0.0f;
             }
     }
 
+    // Byte offsets into a staged record.  They are held in vector registers (the empty asm hides
+    // what the compiler could know about them) so that every LDS read of the unrolled batch is
+    // "register + immediate": no address arithmetic in the loop.
+    const char* const rec_bytes = reinterpret_cast<const char*>(s_rec);
+    uint32_t off_f = 4u * (uint32_t)qx, off_g = 4u * (uint32_t)(kFx + qy), off_u = 4u * (uint32_t)(kFx + kGy);
+    asm volatile("" : "+v"(off_f), "+v"(off_g), "+v"(off_u));
+
+    // Staging role of this lane: Gaussian lane%32 of the batch; lanes 0-31 tabulate F, 32-63 G.
+    const int stage_slot = lane & (kBatch - 1);
+    const bool stage_g = lane >= kBatch;
+    float* const stage_tab = s_rec + stage_slot * kRec + (stage_g ? kFx : 0);
+    const int stage_len = stage_g ? kGy : kFx;
+
     // registers hold the batch that is staged next; loads for it overlap the shading of the current one
     float2 nxy = make_float2(0.f, 0.f);
     float4 nco = make_float4(0.f, 0.f, 0.f, 0.f), nrgb = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (lane < n) {
-        const uint32_t g = point_list[range.x + lane];
+    if (stage_slot < n) {
+        const uint32_t g = point_list[range.x + stage_slot];
         nxy = points_xy[g]; nco = conic_opacity[g]; nrgb = rgb_depth[g];
     }
 
     bool done = false;
-    for (int base = 0; base < n && !done; base += kWave) {
-        const int cnt = min(kWave, n - base);
+    for (int base = 0; base < n && !done; base += kBatch) {
+        const int cnt = min(kBatch, n - base);
         __builtin_amdgcn_wave_barrier();
-        s_a[lane] = make_float4(nxy.x, nxy.y, nco.x, nco.y);
-        s_b[lane] = make_float4(nco.z, nco.w, nrgb.x, nrgb.y);
-        s_c[lane] = nrgb.z;
+        {
+            // conic_opacity = (cx, cy, cz, w) in the units of the exponent (see fgs_preprocess)
+            const float ex = nxy.x - centre_x, ey = nxy.y - centre_y;
+            // offset along the tabulated axis, from the first column (row) of the tile
+            const float e = stage_g ? ey + (float)(kGy / 2) : ex + (float)(kFx / 2);
+            const float curv = stage_g ? nco.z : nco.x;
+            const float lin = nco.y * (stage_g ? ex : ey);
+            const float con = stage_g ? 0.0f : nco.w - (nco.y * ex) * ey;
+#pragma unroll
+            for (int k = 0; k < kTab; k += 4) {
+                float4 t;
+                float* tv = &t.x;
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const float d = e - (float)(k + c);
+                    tv[c] = con + d * (curv * d + lin);
+                }
+                if (k < stage_len) *reinterpret_cast<float4*>(stage_tab + k) = t;
+            }
+            if (stage_g) *reinterpret_cast<float4*>(s_rec + stage_slot * kRec + kFx + kGy) =
+                make_float4(nco.y, nrgb.x, nrgb.y, nrgb.z);
+        }
         __builtin_amdgcn_wave_barrier();
-        if (base + kWave + lane < n) {
-            const uint32_t g = point_list[range.x + base + kWave + lane];
+        if (base + kBatch + stage_slot < n) {
+            const uint32_t g = point_list[range.x + base + kBatch + stage_slot];
             nxy = points_xy[g]; nco = conic_opacity[g]; nrgb = rgb_depth[g];
         }
         // Gaussians go in pairs; the tile-wide stop is tested after each pair (render.cu:394-408)
-        for (int j = 0; j < cnt; j += 2) {
-            {
-                const float4 a = s_a[j], b4 = s_b[j];
-                const float blue = s_c[j];
+        // The table reads of a Gaussian are issued before the Gaussian ahead of it is shaded, so
+        // that a wave does not sit out the LDS latency once per Gaussian.
+        auto fetch = [&](int j) {
+            const int rec = j * kRec * 4;
+            Staged r;
+            r.u = lds_read<float4>(rec_bytes + off_u + rec);
 #pragma unroll
-                for (int s = 0; s < kSub; s++) shade_quad(quad[s], pxf[s], pyf[s], a, b4, blue);
+            for (int c = 0; c < SX; c++) r.f[c] = lds_read<float2>(rec_bytes + off_f + rec + c * 64);
+#pragma unroll
+            for (int c = 0; c < SY; c++) r.g[c] = lds_read<float2>(rec_bytes + off_g + rec + c * 64);
+            return r;
+        };
+        auto shade = [&](const Staged& r) {
+#pragma unroll
+            for (int s = 0; s < kSub; s++) shade_quad(quad[s], xy[s], r.f[s % SX], r.g[s / SX], r.u);
+        };
+        auto all_stopped = [&]() {
+            bool live = false;                      // some pixel of this lane still has T >= 1e-4
+#pragma unroll
+            for (int s = 0; s < kSub; s++) {
+                float m;
+                asm("v_max3_f32 %0, %1, %2, %3" : "=v"(m) : "v"(quad[s].T[0][0]), "v"(quad[s].T[0][1]), "v"(quad[s].T[1][0]));
+                live = live || !(m < 0.0001f) || !(quad[s].T[1][1] < 0.0001f);
             }
-            if (j + 1 >= cnt) break;            // odd tail (render.cu:486-487)
-            {
-                const float4 a = s_a[j + 1], b4 = s_b[j + 1];
-                const float blue = s_c[j + 1];
-#pragma unroll
-                for (int s = 0; s < kSub; s++) shade_quad(quad[s], pxf[s], pyf[s], a, b4, blue);
-            }
-            float tmax = 0.0f;
-#pragma unroll
-            for (int s = 0; s < kSub; s++)
-                tmax = fmaxf(tmax, fmaxf(fmaxf(quad[s].T[0][0], quad[s].T[0][1]), fmaxf(quad[s].T[1][0], quad[s].T[1][1])));
-            if (ballot(!(tmax < 0.0001f)) == 0) { done = true; break; }
-        }
+            return ballot(live) == 0;
+        };
+        // written out for the whole batch so that every record offset is an immediate
+#define FGS_PAIR(J)                                                                   \
+        if ((J) >= cnt) break;                                                        \
+        second = fetch((J) + 1);                                                      \
+        shade(first);                                                                 \
+        if ((J) + 1 >= cnt) break;              /* odd tail (render.cu:486-487) */    \
+        first = fetch(((J) + 2) % kBatch);      /* past the batch: read and dropped */\
+        shade(second);                                                                \
+        if (all_stopped()) { done = true; break; }
+        static_assert(kBatch == 32, "the pairs below cover a batch of 32");
+        Staged first = fetch(0), second;
+        do {
+            FGS_PAIR(0) FGS_PAIR(2) FGS_PAIR(4) FGS_PAIR(6) FGS_PAIR(8) FGS_PAIR(10) FGS_PAIR(12) FGS_PAIR(14)
+            FGS_PAIR(16) FGS_PAIR(18) FGS_PAIR(20) FGS_PAIR(22) FGS_PAIR(24) FGS_PAIR(26) FGS_PAIR(28) FGS_PAIR(30)
+        } while (0);
+#undef FGS_PAIR
     }
 
     // render.cu:59-73
