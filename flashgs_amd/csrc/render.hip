@@ -178,8 +178,13 @@ __global__ __launch_bounds__(kWave) void blend_kernel(
     // registers hold the batch that is staged next; loads for it overlap the shading of the current one
     float2 nxy = make_float2(0.f, 0.f);
     float4 nco = make_float4(0.f, 0.f, 0.f, 0.f), nrgb = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (stage_slot < n) {
-        const uint32_t g = point_list[range.x + stage_slot];
+    // The list index is fetched two batches ahead and the attributes one batch ahead, so that no
+    // wave waits for an index only to start the loads that depend on it.  Positions past the end
+    // of the list are clamped to its last entry: those loads are valid and their result unused.
+    uint32_t g_ahead = 0;
+    if (n > 0) {
+        const uint32_t g = point_list[min(range.x + stage_slot, range.y - 1)];
+        g_ahead = point_list[min(range.x + kBatch + stage_slot, range.y - 1)];
         nxy = points_xy[g]; nco = conic_opacity[g]; nrgb = rgb_depth[g];
     }
 
@@ -210,10 +215,8 @@ __global__ __launch_bounds__(kWave) void blend_kernel(
                 make_float4(nco.y, nrgb.x, nrgb.y, nrgb.z);
         }
         __builtin_amdgcn_wave_barrier();
-        if (base + kBatch + stage_slot < n) {
-            const uint32_t g = point_list[range.x + base + kBatch + stage_slot];
-            nxy = points_xy[g]; nco = conic_opacity[g]; nrgb = rgb_depth[g];
-        }
+        nxy = points_xy[g_ahead]; nco = conic_opacity[g_ahead]; nrgb = rgb_depth[g_ahead];
+        g_ahead = point_list[min(range.x + base + 2 * kBatch + stage_slot, range.y - 1)];
         // Gaussians go in pairs; the tile-wide stop is tested after each pair (render.cu:394-408)
         // The table reads of a Gaussian are issued before the Gaussian ahead of it is shaded, so
         // that a wave does not sit out the LDS latency once per Gaussian.
