@@ -5,12 +5,12 @@
 //
 // Blend layout: one wave64 owns one tile.  A tile is made of 16x16-pixel sub-tiles (1 for 16x16,
 // 2 for 32x16, 4 for 32x32); lane l shades the 2x2 pixel quad at (2*(l%8), 2*(l/8)) of every
-// sub-tile; the quadratic form is evaluated at one pixel of the quad and stepped to the others.  Gaussians are
-// staged 64 at a time into LDS (one per lane: index -> centre, conic+opacity, colour) while the
-// loads of the following batch are already in flight, and the wave walks the batch reading LDS
-// at wave-uniform addresses.  After every second Gaussian one ballot tests whether all pixels of
-// the tile have T < 1e-4, which is the reference's stop rule (render.cu:394-408).  A workgroup is
-// a single wave, so no workgroup barrier is needed anywhere.
+// sub-tile.  Gaussians are staged 32 at a time: the staging lanes tabulate the two one-dimensional
+// parts of the exponent over the tile's columns and rows in LDS, while the loads of the following
+// batch are already in flight; the wave then walks the batch, every lane reading the table
+// entries of its own columns and rows.  After every second Gaussian one ballot tests whether all
+// pixels of the tile have T < 1e-4, which is the reference's stop rule (render.cu:394-408).  A
+// workgroup is a single wave, so no workgroup barrier is needed anywhere.
 #include "fgs_internal.h"
 
 namespace fgs {
