@@ -98,6 +98,19 @@ def test_large_splats_all_tile_sizes(oracle, block):
     assert ref["pre"]["counts"]["candidates"] > 64 * 20
 
 
+@pytest.mark.parametrize("block", [(32, 16), (32, 32)])
+def test_wide_tiles_on_a_frame_with_many_tiles(oracle, block):
+    """5120x2880 has more tiles than the chip holds at once even at 32x32 (160x90 = 14 400):
+    the blend then runs its variant with fewer resident waves."""
+    sc = scenes.config0(n=40_000)
+    cam = sc.cameras[0]
+    scale = 2880 / cam.height
+    cam.width, cam.height = 5120, 2880
+    cam.focal_x *= scale
+    cam.focal_y *= scale
+    _check_frame(oracle, sc, cam, 1 << 22, block=block, bg=(0.1, 0.2, 0.3))
+
+
 def test_anisotropic_splats_near_camera(oracle):
     """Needle-shaped splats close to the camera: the exact ellipse test rejects most candidates."""
     sc = scenes.config4(n=60_000, width=1280, height=720, n_poses=3)
