@@ -24,24 +24,37 @@ __global__ __launch_bounds__(256) void fill_i32_kernel(int* p, size_t n, int v)
     for (; i < n; i += stride) p[i] = v;
 }
 
-// render.cu:9-31, with the tile index checked against the number of tiles
+// render.cu:9-31, with the tile index checked against the number of tiles.  A thread looks at
+// kRangesPerThread pairs, 256 apart so that the loads of a workgroup stay contiguous.
+constexpr int kRangesPerThread = 8;
+
 __global__ __launch_bounds__(256) void tile_ranges_kernel(int L, const uint64_t* __restrict__ keys,
                                                           int2* __restrict__ ranges, uint32_t num_tiles)
 {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= L) return;
-    const uint32_t cur = (uint32_t)(keys[idx] >> 32);
-    if (cur >= num_tiles) return;
-    if (idx == 0) {
-        ranges[cur].x = 0;
-    } else {
-        const uint32_t prev = (uint32_t)(keys[idx - 1] >> 32);
-        if (cur != prev) {
-            if (prev < num_tiles) ranges[prev].y = idx;
-            ranges[cur].x = idx;
+    const long long base = (long long)blockIdx.x * (256 * kRangesPerThread) + threadIdx.x;
+    uint32_t cur[kRangesPerThread], prev[kRangesPerThread];
+#pragma unroll
+    for (int k = 0; k < kRangesPerThread; k++) {
+        const long long idx = base + k * 256;
+        cur[k] = 0; prev[k] = 0;
+        if (idx < L) {
+            cur[k] = (uint32_t)(keys[idx] >> 32);
+            if (idx > 0) prev[k] = (uint32_t)(keys[idx - 1] >> 32);
         }
     }
-    if (idx == L - 1) ranges[cur].y = L;
+#pragma unroll
+    for (int k = 0; k < kRangesPerThread; k++) {
+        const long long idx = base + k * 256;
+        if (idx >= L) break;
+        if (cur[k] >= num_tiles) continue;
+        if (idx == 0) {
+            ranges[cur[k]].x = 0;
+        } else if (cur[k] != prev[k]) {
+            if (prev[k] < num_tiles) ranges[prev[k]].y = (int)idx;
+            ranges[cur[k]].x = (int)idx;
+        }
+        if (idx == L - 1) ranges[cur[k]].y = L;
+    }
 }
 
 // render.cu:54-57
@@ -345,7 +358,9 @@ int ranges_impl(int block_x, int block_y, int num_rendered, int width, int heigh
     if (fill_blocks > 1024) fill_blocks = 1024;
     hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)fill_blocks), dim3(256), 0, st, ranges, words, 0);
     if (num_rendered > 0)
-        hipLaunchKernelGGL(tile_ranges_kernel, dim3((num_rendered + 255) / 256), dim3(256), 0, st,
+        hipLaunchKernelGGL(tile_ranges_kernel,
+                           dim3((unsigned)(((size_t)num_rendered + 256 * kRangesPerThread - 1) / (256 * kRangesPerThread))),
+                           dim3(256), 0, st,
                            num_rendered, keys_sorted, (int2*)ranges,
                            (uint32_t)(num_tiles > 0xffffffffu ? 0xffffffffu : num_tiles));
     return check_hip(hipGetLastError(), who);

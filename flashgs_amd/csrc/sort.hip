@@ -281,21 +281,37 @@ __device__ __forceinline__ int wave_lower_bound(const uint64_t* __restrict__ key
 }
 
 // seg_start[v] = first index whose tile field is >= v, for v in [0, ids]; seg_start[ids] = n.
-// One thread per pair: where the tile field changes, the thread fills the entries of the ids in
-// between (empty ids get the same start as the next non-empty one).  Also clears the flag words.
+// A thread looks at kStartsPerThread pairs, 256 apart so that the loads of a workgroup stay
+// contiguous: where the tile field changes, it fills the entries of the ids in between (empty ids
+// get the same start as the next non-empty one).  Also clears the flag words and list counters.
+constexpr int kStartsPerThread = 8;
+
 __global__ __launch_bounds__(256) void segment_starts_kernel(const uint64_t* __restrict__ keys, int n, uint32_t tile_mask,
                                                              uint32_t ids, int* __restrict__ seg_start,
                                                              uint32_t* __restrict__ seg_flags, uint32_t* __restrict__ seg_counts)
 {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if ((uint32_t)i < (ids + 31) / 32) seg_flags[i] = 0;
-    if (i < 2) seg_counts[i] = 0;
-    if (i >= n) return;
-    const uint32_t cur = (uint32_t)(keys[i] >> 32) & tile_mask;
-    const uint32_t first = i == 0 ? 0u : ((uint32_t)(keys[i - 1] >> 32) & tile_mask) + 1u;
-    for (uint32_t v = first; v <= cur; v++) seg_start[v] = i;      // empty loop when the field repeats
-    if (i == n - 1)
-        for (uint32_t v = cur + 1; v <= ids; v++) seg_start[v] = n;
+    const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
+    for (uint32_t w = gid; w < (ids + 31) / 32; w += gridDim.x * blockDim.x) seg_flags[w] = 0;
+    if (gid < 2) seg_counts[gid] = 0;
+    const long long base = (long long)blockIdx.x * (256 * kStartsPerThread) + threadIdx.x;
+    uint32_t cur[kStartsPerThread], before[kStartsPerThread];
+#pragma unroll
+    for (int k = 0; k < kStartsPerThread; k++) {
+        const long long i = base + k * 256;
+        cur[k] = 0; before[k] = 0;
+        if (i < n) {
+            cur[k] = (uint32_t)(keys[i] >> 32) & tile_mask;
+            before[k] = i == 0 ? 0u : ((uint32_t)(keys[i - 1] >> 32) & tile_mask) + 1u;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kStartsPerThread; k++) {
+        const long long i = base + k * 256;
+        if (i >= n) break;
+        for (uint32_t v = before[k]; v <= cur[k]; v++) seg_start[v] = (int)i;     // empty loop when the field repeats
+        if (i == n - 1)
+            for (uint32_t v = cur[k] + 1; v <= ids; v++) seg_start[v] = n;
+    }
 }
 
 // One stable counting pass of a segment over bits shift..shift+7 of the sort word, by the kWaves
@@ -811,7 +827,7 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         if (ids <= kMaxTableIds) {
             seg_start = (int*)(list_sorting_space + ws.seg_start);
             seg_flags = (uint32_t*)(list_sorting_space + ws.seg_flags);
-            const unsigned blocks = (unsigned)(((size_t)(n > (int)(ids / 32 + 1) ? n : (int)(ids / 32 + 1)) + 255) / 256);
+            const unsigned blocks = (unsigned)(((size_t)n + 256 * kStartsPerThread - 1) / (256 * kStartsPerThread));
             hipLaunchKernelGGL(segment_starts_kernel, dim3(blocks), dim3(256), 0, st,
                                (const uint64_t*)gaussian_keys_sorted, n, tile_mask, ids, seg_start, seg_flags,
                                (uint32_t*)(list_sorting_space + ws.seg_lists));
