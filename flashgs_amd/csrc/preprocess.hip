@@ -189,40 +189,60 @@ __device__ __forceinline__ void sh_to_rgb(const float* __restrict__ sh, float px
                     C3_3 = 0.3731763325901154f, C3_4 = -0.4570457994644658f, C3_5 = 1.445305721320277f,
                     C3_6 = -0.5900435899266435f;
 
-    // 48 floats = 12 aligned 16-byte loads (the record is 192 bytes)
-    float v[48];
+    // 48 floats = 12 aligned 16-byte loads (the record is 192 bytes), taken in four groups of
+    // four coefficients per channel so that only 12 of them are live at a time: the sums below
+    // run in coefficient order, so splitting them changes no result.
     const float4* src = reinterpret_cast<const float4*>(sh);
+    float v[12];
+    auto load_group = [&](int g) {
 #pragma unroll
-    for (int q = 0; q < 12; q++) {
-        float4 f = src[q];
-        v[4 * q + 0] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
-    }
-
+        for (int q = 0; q < 3; q++) {
+            float4 f = src[3 * g + q];
+            v[4 * q + 0] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
+        }
+    };
+    load_group(0);
     float dx = px - cam.campos[0], dy = py - cam.campos[1], dz = pz - cam.campos[2];
     float l2 = dx * dx + dy * dy + dz * dz;
     float inv = 1.0f / __builtin_sqrtf(l2);
     float x = dx * inv, y = dy * inv, z = dz * inv;
     float xx = x * x, yy = y * y, zz = z * z;
     float xy = x * y, yz = y * z, xz = x * z;
+    float res[3];
 #pragma unroll
-    for (int ch = 0; ch < 3; ch++) {
-        float res = C0 * v[ch] + 0.5f;
-        res = res - C1 * y * v[3 + ch] + C1 * z * v[6 + ch] - C1 * x * v[9 + ch];
-        res = res +
-              C2_0 * xy * v[12 + ch] +
-              C2_1 * yz * v[15 + ch] +
-              C2_2 * (2.0f * zz - xx - yy) * v[18 + ch] +
-              C2_3 * xz * v[21 + ch] +
-              C2_4 * (xx - yy) * v[24 + ch];
-        res = res +
-              C3_0 * y * (3.0f * xx - yy) * v[27 + ch] +
-              C3_1 * xy * z * v[30 + ch] +
-              C3_2 * y * (4.0f * zz - xx - yy) * v[33 + ch] +
-              C3_3 * z * (2.0f * zz - 3.0f * xx - 3.0f * yy) * v[36 + ch] +
-              C3_4 * x * (4.0f * zz - xx - yy) * v[39 + ch] +
-              C3_5 * z * (xx - yy) * v[42 + ch] +
-              C3_6 * x * (xx - 3.0f * yy) * v[45 + ch];
-        rgb[ch] = max_f(res, 0.0f);
+    for (int ch = 0; ch < 3; ch++) {        // coefficients 0-3
+        float r = C0 * v[ch] + 0.5f;
+        res[ch] = r - C1 * y * v[3 + ch] + C1 * z * v[6 + ch] - C1 * x * v[9 + ch];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    load_group(1);
+#pragma unroll
+    for (int ch = 0; ch < 3; ch++)          // coefficients 4-7
+        res[ch] = res[ch] +
+                  C2_0 * xy * v[0 + ch] +
+                  C2_1 * yz * v[3 + ch] +
+                  C2_2 * (2.0f * zz - xx - yy) * v[6 + ch] +
+                  C2_3 * xz * v[9 + ch];
+    __builtin_amdgcn_sched_barrier(0);
+    load_group(2);
+#pragma unroll
+    for (int ch = 0; ch < 3; ch++) {        // coefficients 8-11
+        float r = res[ch] + C2_4 * (xx - yy) * v[0 + ch];
+        res[ch] = r +
+                  C3_0 * y * (3.0f * xx - yy) * v[3 + ch] +
+                  C3_1 * xy * z * v[6 + ch] +
+                  C3_2 * y * (4.0f * zz - xx - yy) * v[9 + ch];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    load_group(3);
+#pragma unroll
+    for (int ch = 0; ch < 3; ch++) {        // coefficients 12-15
+        float r = res[ch] +
+                  C3_3 * z * (2.0f * zz - 3.0f * xx - 3.0f * yy) * v[0 + ch] +
+                  C3_4 * x * (4.0f * zz - xx - yy) * v[3 + ch] +
+                  C3_5 * z * (xx - yy) * v[6 + ch] +
+                  C3_6 * x * (xx - 3.0f * yy) * v[9 + ch];
+        rgb[ch] = max_f(r, 0.0f);
     }
 }
 
