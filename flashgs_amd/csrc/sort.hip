@@ -148,7 +148,10 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
     int n, int shift, int nbits,
     const uint32_t* __restrict__ start)          // [blocks][kBins] from offsets_kernel
 {
-    __shared__ uint32_t s_count[kSortWaves][kBins];   // per-wave digit counts, then per-wave digit offsets
+    // per-wave digit counts, then per-wave digit offsets: at most kTile, so 16 bits do, and with
+    // them the workgroup's LDS stays under a third of the CU's (three resident workgroups, not two)
+    __shared__ uint16_t s_count[kSortWaves][kBins];
+    static_assert(kTile <= 65535, "s_count holds 16-bit counts");
     __shared__ uint32_t s_bin_start[kBins];           // where each digit starts in the ranked block
     __shared__ uint32_t s_global[kBins];              // destination of ranked slot p with digit d: s_global[d] + p
     __shared__ uint32_t s_wave_sum[kSortWaves];
@@ -200,7 +203,7 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
         uint32_t before = 0;
         if (valid && below == 0) {      // lowest lane of each group updates the wave's counter
             before = s_count[wave][d];
-            s_count[wave][d] = before + (uint32_t)__popcll(peers);
+            s_count[wave][d] = (uint16_t)(before + (uint32_t)__popcll(peers));
         }
         const int leader = valid ? __ffsll((long long)peers) - 1 : lane;
         before = (uint32_t)__shfl((int)before, leader);
@@ -215,7 +218,7 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
 #pragma unroll
     for (int w = 0; w < kSortWaves; w++) {
         const uint32_t c = s_count[w][d];
-        s_count[w][d] = total;
+        s_count[w][d] = (uint16_t)total;
         total += c;
     }
     uint32_t incl = wave_inclusive_sum(total);
