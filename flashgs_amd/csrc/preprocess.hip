@@ -248,16 +248,22 @@ __device__ __forceinline__ void sh_to_rgb(const float* __restrict__ sh, float px
 
 // ---- chained scan over workgroups ---------------------------------------------------------------
 //
-// status word: [63:34] epoch of the launch, [33:32] state, [31:0] count.
-// A word whose epoch differs from the running launch's reads as "nothing published yet", so the
-// array never has to be cleared between launches.
+// status word: [33:32] state, [31:0] count; 0 = nothing published yet.
+// The scratch holds a control word and two status arrays.  A launch works in the array the
+// control word names and clears the other one, which the launch after it will use; its last
+// workgroup flips the control word when its own walk back is over.  That walk ends only when
+// every earlier workgroup has published, i.e. after all of them have read the control word, so
+// no workgroup of this launch can see the flipped value; the next launch (same stream, or
+// otherwise ordered after this one) starts from it.  Nothing on the host changes from launch to
+// launch, so a captured launch can be replayed.
+constexpr int kControlWords = 8;          // control word + padding in front of the two arrays
 constexpr uint64_t kStateAggregate = 1;   // count of this workgroup only
 constexpr uint64_t kStatePrefix = 2;      // count of this workgroup and all before it
 constexpr uint64_t kStatePoison = 3;      // like kStatePrefix, but a predecessor never published
 
-__device__ __forceinline__ uint64_t pack_status(uint32_t epoch, uint64_t state, uint32_t value)
+__device__ __forceinline__ uint64_t pack_status(uint64_t state, uint32_t value)
 {
-    return ((uint64_t)epoch << 34) | (state << 32) | (uint64_t)value;
+    return (state << 32) | (uint64_t)value;
 }
 
 __device__ __forceinline__ void publish(uint64_t* slot, uint64_t word)
@@ -280,7 +286,7 @@ __device__ __forceinline__ uint64_t peek(const uint64_t* slot)
 // itself; the wait is bounded so that every wave of the grid exits whatever happens.
 constexpr int kLookAhead = 4;
 
-__device__ __forceinline__ uint32_t look_back(const uint64_t* status, int ticket, uint32_t epoch, bool* failed)
+__device__ __forceinline__ uint32_t look_back(const uint64_t* status, int ticket, bool* failed)
 {
     const int lane = lane_id();
     uint32_t sum = 0;
@@ -301,7 +307,7 @@ __device__ __forceinline__ uint32_t look_back(const uint64_t* status, int ticket
             uint64_t closing;        // lanes holding a prefix (or poison) word
             for (;;) {
                 state = 0;
-                if (j >= 0 && (uint32_t)(word >> 34) == epoch) state = (uint32_t)(word >> 32) & 3u;
+                if (j >= 0) state = (uint32_t)(word >> 32) & 3u;
                 const uint64_t pending = ballot(j >= 0 && state == 0);
                 closing = ballot(state >= kStatePrefix);
                 const uint64_t need = closing ? ((closing & (~closing + 1)) << 1) - 1 : ~0ull;
@@ -337,8 +343,8 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     uint32_t* __restrict__ values,
     int* __restrict__ curr_offset,
     int64_t capacity,            // <= 0: unchecked
-    uint64_t* __restrict__ status,
-    uint32_t epoch,
+    uint64_t* __restrict__ scratch,        // control word, then two status arrays of status_capacity words
+    int status_capacity,
     int num_blocks)
 {
     __shared__ uint32_t s_wave_total[kWavesPerBlock];
@@ -364,6 +370,14 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     // for it (and the wait is bounded in any case).
     const int ticket = (int)blockIdx.x;
     const int idx = ticket * kBlock + tid;
+    // this launch's status array; the other one is cleared for the launch that follows
+    const uint32_t which = (uint32_t)peek(scratch) & 1u;
+    uint64_t* const status = scratch + kControlWords + (size_t)which * status_capacity;
+    {
+        uint64_t* const other = scratch + kControlWords + (size_t)(which ^ 1u) * status_capacity;
+        for (long long w = ticket + (long long)tid * num_blocks; w < status_capacity; w += (long long)kBlock * num_blocks)
+            other[w] = 0;
+    }
     // tile coordinates travel in 12 bits each and tile indices in 26 when candidates are laid flat
     const bool pack_ok = cam.gx <= 4096 && cam.gy <= 4096 && (long long)cam.gx * cam.gy <= (1 << 26);
 
@@ -571,7 +585,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
 
     // The workgroup's count is published right away; the wait for the counts of earlier
     // workgroups comes after the colour work below, when they have long been published.
-    if (tid == 0 && ticket != 0) publish(status + ticket, pack_status(epoch, kStateAggregate, block_total));
+    if (tid == 0 && ticket != 0) publish(status + ticket, pack_status(kStateAggregate, block_total));
 
     // ---- attributes of Gaussians that emit a key (preprocess.cu:411-417) ----
     if (count > 0) {
@@ -588,12 +602,16 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         bool timed_out = false;
         uint32_t excl;
         if (ticket == 0) excl = (uint32_t)*curr_offset;     // the caller's starting offset (example.py:69 zeroes it)
-        else excl = look_back(status, ticket, epoch, &timed_out);
+        else excl = look_back(status, ticket, &timed_out);
         if (lane == 0) {
-            publish(status + ticket, pack_status(epoch, timed_out ? kStatePoison : kStatePrefix, excl + block_total));
+            publish(status + ticket, pack_status(timed_out ? kStatePoison : kStatePrefix, excl + block_total));
             s_block_base = excl;
-            // only the last workgroup writes the counter; a poisoned chain yields a negative count
-            if (ticket == num_blocks - 1) *curr_offset = timed_out ? -2147483647 - 1 : (int)(excl + block_total);
+            // only the last workgroup writes the counter (a poisoned chain yields a negative count)
+            // and hands the other status array to the next launch
+            if (ticket == num_blocks - 1) {
+                *curr_offset = timed_out ? -2147483647 - 1 : (int)(excl + block_total);
+                publish(scratch, (uint64_t)(which ^ 1u));
+            }
         }
     }
     __syncthreads();
@@ -690,9 +708,8 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
 // ---- per-device scratch for the chained scan ------------------------------------------------------
 
 struct Scratch {
-    uint64_t* status = nullptr;     // one word per workgroup
-    size_t status_words = 0;
-    uint32_t epoch = 0;
+    uint64_t* words = nullptr;      // control word (+ padding), then two status arrays
+    size_t capacity = 0;            // workgroups each status array holds
 };
 
 constexpr int kMaxDevices = 64;
@@ -702,31 +719,23 @@ std::mutex g_mutex;
 int acquire_scratch(int device, int num_blocks, hipStream_t stream, Scratch** out)
 {
     Scratch& s = g_scratch[device];
-    if (s.status_words < (size_t)num_blocks) {
-        // the stream may still be reading the old array: drain it before the swap
+    if (s.capacity < (size_t)num_blocks) {
+        // the stream may still be reading the old arrays: drain it before the swap
         FGS_HIP_TRY(hipStreamSynchronize(stream));
-        if (s.status) FGS_HIP_TRY(hipFree(s.status));
-        s.status = nullptr;
-        s.status_words = 0;
-        size_t words = 1;
-        while (words < (size_t)num_blocks) words <<= 1;
-        if (words < 4096) words = 4096;
-        if (hipMalloc((void**)&s.status, words * sizeof(uint64_t)) != hipSuccess) {
+        if (s.words) FGS_HIP_TRY(hipFree(s.words));
+        s.words = nullptr;
+        s.capacity = 0;
+        size_t cap = 4096;
+        while (cap < (size_t)num_blocks) cap <<= 1;
+        const size_t bytes = (kControlWords + 2 * cap) * sizeof(uint64_t);
+        if (hipMalloc((void**)&s.words, bytes) != hipSuccess) {
             (void)hipGetLastError();
-            return fail(FGS_E_NOMEM, "cannot allocate %zu bytes of scan status", words * sizeof(uint64_t));
+            return fail(FGS_E_NOMEM, "cannot allocate %zu bytes of scan status", bytes);
         }
-        FGS_HIP_TRY(hipMemset(s.status, 0, words * sizeof(uint64_t)));
+        FGS_HIP_TRY(hipMemset(s.words, 0, bytes));
         FGS_HIP_TRY(hipDeviceSynchronize());
-        s.status_words = words;
-        s.epoch = 0;
+        s.capacity = cap;
     }
-    if (s.epoch >= (1u << 30) - 1) {   // epoch field is 30 bits wide: start over on a clean array
-        FGS_HIP_TRY(hipStreamSynchronize(stream));
-        FGS_HIP_TRY(hipMemset(s.status, 0, s.status_words * sizeof(uint64_t)));
-        FGS_HIP_TRY(hipDeviceSynchronize());
-        s.epoch = 0;
-    }
-    s.epoch++;
     *out = &s;
     return FGS_OK;
 }
@@ -828,6 +837,6 @@ extern "C" int fgs_preprocess(int P,
     hipLaunchKernelGGL(preprocess_kernel, dim3(num_blocks), dim3(kBlock), 0, st,
                        P, positions, shs, opacities, cov3Ds, cam, points_xy, rgb_depth, conic_opacity,
                        gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset, key_capacity,
-                       s->status, s->epoch, num_blocks);
+                       s->words, (int)s->capacity, num_blocks);
     return check_hip(hipGetLastError(), "preprocess_kernel launch");
 }

@@ -166,6 +166,51 @@ def test_start_offset_and_capacity_guard(oracle):
     assert np.all(gp.u64(keys)[cap:] == 0) and np.all(values.cpu().numpy()[cap:] == -1)   # nothing past the capacity
 
 
+def test_preprocess_replayed_from_a_captured_graph():
+    """fgs_preprocess keeps no per-launch state on the host, so a captured launch can be replayed:
+    every replay (with eager launches of other sizes in between) gives the eager result."""
+    import gpu_pipeline as gp
+    import torch
+    from flashgs_amd import cabi
+    sc = scenes.config0(n=70_000)
+    cam = sc.cameras[0]
+    sd = gp.SceneOnDevice(sc)
+    cap = 1 << 20
+    eager = gp.preprocess(sd, cam, cap)
+    K = eager["num_rendered"]
+    ref_keys = gp.u64(eager["keys"])[:K].copy()
+    ref_vals = gp.u32(eager["values"])[:K].copy()
+    n = sd.n
+    xy = torch.zeros((n, 2), device=gp.DEV); rgb = torch.zeros((n, 4), device=gp.DEV); co = torch.zeros((n, 4), device=gp.DEV)
+    keys = torch.zeros(cap, device=gp.DEV, dtype=torch.int64)
+    values = torch.zeros(cap, device=gp.DEV, dtype=torch.int32)
+    off = torch.zeros(1, device=gp.DEV, dtype=torch.int32)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        off.zero_()                     # a fill kernel, not a memset node
+        cabi.preprocess(n, sd.position.data_ptr(), sd.shs.data_ptr(), sd.opacity.data_ptr(), sd.cov3d.data_ptr(),
+                        cam.width, cam.height, 16, 16, cam.position, cam.rotation, cam.focal_x, cam.focal_y,
+                        cam.zFar, cam.zNear, xy.data_ptr(), rgb.data_ptr(), co.data_ptr(),
+                        keys.data_ptr(), values.data_ptr(), off.data_ptr(), cap, torch.cuda.current_stream().cuda_stream)
+    small = gp.SceneOnDevice(scenes.config0(n=3000))
+    for replay in range(4):
+        keys.zero_(); values.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(off.cpu()[0]) == K, "replay %d" % replay
+        assert np.array_equal(gp.u64(keys)[:K], ref_keys), "replay %d" % replay
+        assert np.array_equal(gp.u32(values)[:K], ref_vals), "replay %d" % replay
+        for name, t in (("points_xy", xy), ("rgb_depth", rgb), ("conic_opacity", co)):
+            vis = np.unique(ref_vals)
+            assert np.array_equal(gp.bits(t.cpu().numpy()[vis]), gp.bits(eager[name].cpu().numpy()[vis])), name
+        # eager launches of another size between the replays
+        for _ in range(replay + 1):
+            gp.preprocess(small, cam, 1 << 16)
+        torch.cuda.synchronize()
+
+
 def test_repeated_frames_are_deterministic():
     import gpu_pipeline as gp
     sc = scenes.config0(n=50_000)
