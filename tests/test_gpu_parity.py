@@ -211,6 +211,48 @@ def test_preprocess_replayed_from_a_captured_graph():
         torch.cuda.synchronize()
 
 
+def test_sort_and_render_replayed_from_a_captured_graph():
+    """The other two stages keep no state at all between calls: sort + render of a fixed pair count,
+    captured once and replayed with eager work in between, reproduce the eager image."""
+    import gpu_pipeline as gp
+    import torch
+    from flashgs_amd import cabi
+    sc = scenes.config0(n=60_000)
+    cam = sc.cameras[0]
+    sd = gp.SceneOnDevice(sc)
+    pre = gp.preprocess(sd, cam, 1 << 20)
+    K = pre["num_rendered"]
+    ks_e, vs_e = gp.sort(K, cam.width, cam.height, pre["keys"], pre["values"])
+    rg_e, u8_e, _ = gp.render(K, cam.width, cam.height, pre["points_xy"], pre["rgb_depth"], pre["conic_opacity"],
+                              ks_e, vs_e, (0.2, 0.4, 0.6), f32=False)
+    size = cabi.get_sort_buffer_size(K)
+    space = torch.zeros(size, device=gp.DEV, dtype=torch.int8)
+    ks = torch.zeros(K, device=gp.DEV, dtype=torch.int64)
+    vs = torch.zeros(K, device=gp.DEV, dtype=torch.int32)
+    gx, gy = (cam.width + 15) // 16, (cam.height + 15) // 16
+    ranges = torch.zeros((gx * gy, 2), device=gp.DEV, dtype=torch.int32)
+    out = torch.zeros((cam.height, cam.width, 3), device=gp.DEV, dtype=torch.uint8)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        st = torch.cuda.current_stream().cuda_stream
+        cabi.sort_gaussian(K, cam.width, cam.height, 16, 16, space.data_ptr(), size,
+                           pre["keys"].data_ptr(), pre["values"].data_ptr(), ks.data_ptr(), vs.data_ptr(), st)
+        cabi.render(16, 16, K, cam.width, cam.height, pre["points_xy"].data_ptr(), pre["rgb_depth"].data_ptr(),
+                    pre["conic_opacity"].data_ptr(), ks.data_ptr(), vs.data_ptr(), ranges.data_ptr(), (0.2, 0.4, 0.6),
+                    out.data_ptr(), st)
+    for replay in range(3):
+        ks.zero_(); vs.zero_(); out.zero_(); ranges.fill_(-3); space.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(gp.u64(ks), gp.u64(ks_e)[:K]), "replay %d" % replay
+        assert np.array_equal(gp.u32(vs), gp.u32(vs_e)[:K]), "replay %d" % replay
+        assert torch.equal(ranges, rg_e) and torch.equal(out, u8_e), "replay %d" % replay
+        gp.sort(1000, cam.width, cam.height, pre["keys"], pre["values"])       # eager work of another size
+        torch.cuda.synchronize()
+
+
 def test_repeated_frames_are_deterministic():
     import gpu_pipeline as gp
     sc = scenes.config0(n=50_000)
