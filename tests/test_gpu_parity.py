@@ -331,11 +331,16 @@ def test_ranges_kernel_against_searchsorted():
         assert np.array_equal(rg.cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("config", [1, 2])
+@pytest.mark.parametrize("config", [1, 2, 4])
 def test_full_size_configs(oracle, config):
-    """The 1080p / 1M and the 4K / 3M configurations end to end against the oracle."""
+    """The 1080p / 1M, the 4K / 3M and (first and a later pose of) the 2M orbit configurations end to
+    end against the oracle.  The orbit has needle-shaped splats next to the camera whose candidate
+    rectangles cover the screen: most of its candidates are rejected by the exact tile test."""
     sc = scenes.make(config)
-    _check_frame(oracle, sc, sc.cameras[0], 1 << 24)
+    for cam in (sc.cameras[0], sc.cameras[len(sc.cameras) // 2]) if config == 4 else (sc.cameras[0],):
+        ref = _check_frame(oracle, sc, cam, 1 << 24)
+        if config == 4:
+            assert ref["pre"]["counts"]["candidates"] > 3 * ref["K"]
 
 
 def _sort_case(tile, depth_bits, W, H, junk=None, seed=0):
