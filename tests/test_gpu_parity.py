@@ -111,6 +111,49 @@ def test_wide_tiles_on_a_frame_with_many_tiles(oracle, block):
     _check_frame(oracle, sc, cam, 1 << 22, block=block, bg=(0.1, 0.2, 0.3))
 
 
+def test_degenerate_inputs_match_the_oracle(oracle):
+    """NaN / infinite / zero / enormous entries in every input tensor: the kernels must neither fault
+    nor disagree with the oracle about which keys such Gaussians emit (the float->int conversions
+    saturate and map NaN to 0 on both sides)."""
+    sc = scenes.config0(n=20_000)
+    rng = np.random.default_rng(5)
+    bad = [np.nan, np.inf, -np.inf, 0.0, 1e30, -1e30, 1e-30]
+    for arr in (sc.position, sc.opacity, sc.cov3d, sc.shs):
+        flat = arr.reshape(-1)
+        where = rng.choice(flat.size, 300, replace=False)
+        flat[where] = rng.choice(bad, where.size).astype(np.float32)
+    sc.cov3d[100:140] = 0.0                      # degenerate covariances
+    sc.cov3d[200:220] *= 1e6                     # splats far larger than the screen
+    sc.opacity[300:320] = 1.0
+    sc.opacity[320:340] = 1.0 / 255.0
+    import gpu_pipeline as gp
+    cam = sc.cameras[0]
+    cap = 1 << 22
+    pre = oracle.preprocess(sc.position, sc.shs, sc.opacity, sc.cov3d, cam.width, cam.height, 16, 16,
+                            cam.position, cam.rotation, cam.focal_x, cam.focal_y, cam.zFar, cam.zNear, cap)
+    K = pre["num_rendered"]
+    assert 0 < K < cap
+    got = gp.preprocess(gp.SceneOnDevice(sc), cam, cap)
+    assert got["num_rendered"] == K
+    assert np.array_equal(gp.u64(got["keys"])[:K], pre["keys"][:K])
+    assert np.array_equal(gp.u32(got["values"])[:K], pre["values"][:K])
+    vis = np.unique(pre["values"][:K])
+    for name in ("points_xy", "conic_opacity", "rgb_depth"):
+        a, b = got[name].cpu().numpy()[vis], pre[name][vis]
+        # bit-exact, except that a NaN may carry another sign or payload
+        same = (gp.bits(a) == gp.bits(b)) | (np.isnan(a) & np.isnan(b))
+        rows = np.flatnonzero(~same.all(axis=1))
+        assert rows.size == 0, "%s: %d rows differ, first Gaussian %d: %r vs %r" % (
+            name, rows.size, vis[rows[0]], a[rows[0]], b[rows[0]])
+    ks, vs = gp.sort(K, cam.width, cam.height, got["keys"], got["values"])
+    oks, ovs = oracle.sort(K, cam.width, cam.height, 16, 16, pre["keys"], pre["values"])
+    assert np.array_equal(gp.u64(ks)[:K], oks) and np.array_equal(gp.u32(vs)[:K], ovs)
+    # the image may hold NaN where a NaN colour was blended: only require that the blend runs
+    rg, u8, _ = gp.render(K, cam.width, cam.height, got["points_xy"], got["rgb_depth"], got["conic_opacity"],
+                          ks, vs, (0, 0, 0), f32=False)
+    assert np.array_equal(rg.cpu().numpy(), oracle.ranges(K, oks, rg.shape[0]))
+
+
 def test_anisotropic_splats_near_camera(oracle):
     """Needle-shaped splats close to the camera: the exact ellipse test rejects most candidates."""
     sc = scenes.config4(n=60_000, width=1280, height=720, n_poses=3)
