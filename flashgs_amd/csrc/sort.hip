@@ -39,6 +39,12 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // segment workgroup searches for its own bounds.
 constexpr uint32_t kMaxTableIds = 1u << 20;
 
+// The ids of the longer segments are listed per size class in kListShards separate lists (each
+// with its own counter, a workgroup appends to the list of its index modulo kListShards): one
+// shared counter would serialise thousands of atomic additions on one address.
+constexpr int kListShards = 32;
+constexpr int kListClasses = 3;
+
 struct Workspace {
     size_t alt_keys, alt_values, hist, chunk_sums, seg_start, seg_flags, seg_lists, total;
     int tiles, chunk, chunks;       // chunks of `chunk` histogram rows each
@@ -56,9 +62,10 @@ Workspace workspace_for(int n)
     w.chunk_sums = w.hist + (size_t)w.tiles * kBins * 4;
     w.seg_start = w.chunk_sums + (size_t)w.chunks * kBins * 4;
     w.seg_flags = w.seg_start + align_up(((size_t)kMaxTableIds + 1) * 4, 256);
-    // counters (64 words), then the ids of the medium and of the large segments
     w.seg_lists = w.seg_flags + kMaxTableIds / 8;
-    w.total = w.seg_lists + 256 + ((size_t)n / 1024 + 2) * 4 + ((size_t)n / 4096 + 2) * 4;
+    // counters (kListClasses * kListShards words), then per class kListShards lists, each able to
+    // hold every segment of its class
+    w.total = w.seg_lists + 512 + (size_t)kListShards * (((size_t)n / 512 + 2) + ((size_t)n / 1024 + 2) + ((size_t)n / 4096 + 2)) * 4;
     return w;
 }
 
@@ -295,7 +302,7 @@ __global__ __launch_bounds__(256) void segment_starts_kernel(const uint64_t* __r
 {
     const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
     for (uint32_t w = gid; w < (ids + 31) / 32; w += gridDim.x * blockDim.x) seg_flags[w] = 0;
-    if (gid < 2) seg_counts[gid] = 0;
+    if (gid < (uint32_t)(kListClasses * kListShards)) seg_counts[gid] = 0;
     const long long base = (long long)blockIdx.x * (256 * kStartsPerThread) + threadIdx.x;
     uint32_t cur[kStartsPerThread], before[kStartsPerThread];
 #pragma unroll
@@ -471,7 +478,7 @@ template <int kWaves, int kCap, int kIds>
 __global__ __launch_bounds__(kWaves * kWave) void segment_sort_kernel(
     uint64_t* __restrict__ keys, uint32_t* __restrict__ values, int n, uint32_t tile_mask, int min_len, uint32_t ids,
     const int* __restrict__ seg_start, uint32_t* __restrict__ seg_flags,
-    const uint32_t* __restrict__ list, const uint32_t* __restrict__ list_count)
+    const uint32_t* __restrict__ list, const uint32_t* __restrict__ list_count, uint32_t list_cap)
 {
     __shared__ uint32_t s_k[2][kCap];
     __shared__ uint32_t s_v[2][kCap];
@@ -498,10 +505,11 @@ __global__ __launch_bounds__(kWaves * kWave) void segment_sort_kernel(
         return;
     }
 
-    if (list) {      // the segments of this class were listed: deal them out round-robin
-        const uint32_t count = *list_count;
-        for (uint32_t i = blockIdx.x; i < count; i += gridDim.x) {
-            const uint32_t v = list[i];
+    if (list) {      // the segments of this class were listed: deal them out round-robin, shard by shard
+        const uint32_t shard = blockIdx.x % kListShards;
+        const uint32_t count = list_count[shard];
+        for (uint32_t i = blockIdx.x / kListShards; i < count; i += gridDim.x / kListShards) {
+            const uint32_t v = list[(size_t)shard * list_cap + i];
             sort_segment_lds<kWaves, kCap>(keys, values, v, seg_start[v], seg_start[v + 1], seg_flags,
                                            s_k, s_v, s_cnt, s_wave_sum, &s_flag);
         }
@@ -524,30 +532,100 @@ __global__ __launch_bounds__(kWaves * kWave) void segment_sort_kernel(
     }
 }
 
-// Segment sort by a single wave that keeps its pairs in registers: lane l holds pairs
-// l, l+64, ... (kT of them), LDS is only the scatter target of each pass and the 256 digit
-// counters.  For segments with min_len < length <= 64*kT.  Everything is unrolled over the kT
-// pairs of a lane, so the ballot work of different pairs overlaps with the LDS round trips of the
-// running digit counters.
+// x of lane (l ^ kJ).  Within a row of 16 lanes the exchange is a data-parallel-primitive move
+// (no LDS traffic); across rows it goes through the lane crossbar.
+template <int kJ>
+__device__ __forceinline__ uint32_t from_lane_xor(uint32_t x)
+{
+    constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E, kQuadReverse = 0x1B, kRowHalfMirror = 0x141, kRowRor8 = 0x128;
+    if (kJ == 1) return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, kQuadXor1, 0xf, 0xf, true);
+    if (kJ == 2) return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, kQuadXor2, 0xf, 0xf, true);
+    if (kJ == 4) {      // reverse the 8 lanes, then each quad: lane l reads lane l ^ 4
+        const int t = __builtin_amdgcn_mov_dpp((int)x, kRowHalfMirror, 0xf, 0xf, true);
+        return (uint32_t)__builtin_amdgcn_mov_dpp(t, kQuadReverse, 0xf, 0xf, true);
+    }
+    if (kJ == 8) return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, kRowRor8, 0xf, 0xf, true);
+    return (uint32_t)__shfl_xor((int)x, kJ);
+}
+
+template <int kJ>
+__device__ __forceinline__ uint64_t from_lane_xor64(uint64_t x)
+{
+    return ((uint64_t)from_lane_xor<kJ>((uint32_t)(x >> 32)) << 32) | from_lane_xor<kJ>((uint32_t)x);
+}
+
+// The network over kT register slots of every lane, 64 * kT elements.  The merge width k runs
+// in a loop; the compare distances j are written out, so the code holds every exchange pattern
+// once whatever the number of stages.
 template <int kT>
-__device__ __forceinline__ void sort_segment_wave(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
-                                                  uint32_t v, int lo, int hi, uint32_t* __restrict__ seg_flags,
-                                                  uint32_t* s_k, uint32_t* s_v, uint32_t* cnt)
+__device__ __forceinline__ void bitonic_network(uint64_t (&c)[kT], int lane)
+{
+    constexpr int n = kT * kWave;
+#pragma unroll 1
+    for (int k = 2; k <= n; k <<= 1) {
+        bool ascending[kT];                 // element t*64 + lane sits in an ascending run of width k
+#pragma unroll
+        for (int t = 0; t < kT; t++) ascending[t] = ((t * kWave + lane) & k) == 0;
+#pragma unroll
+        for (int j = n / 2; j > 0; j >>= 1) {
+            if (j >= k) continue;
+            if (j >= kWave) {
+                const int jt = j / kWave;
+#pragma unroll
+                for (int t = 0; t < kT; t++) {
+                    if ((t & jt) != 0) continue;
+                    const int t2 = t | jt;
+                    const bool swap = (c[t] > c[t2]) == ascending[t];
+                    const uint64_t a = swap ? c[t2] : c[t], b = swap ? c[t] : c[t2];
+                    c[t] = a; c[t2] = b;
+                }
+            } else {
+                const bool lower = (lane & j) == 0;
+#pragma unroll
+                for (int t = 0; t < kT; t++) {
+                    const uint64_t mine = c[t];
+                    const uint64_t other = j == 1 ? from_lane_xor64<1>(mine) : j == 2 ? from_lane_xor64<2>(mine)
+                                         : j == 4 ? from_lane_xor64<4>(mine) : j == 8 ? from_lane_xor64<8>(mine)
+                                         : j == 16 ? from_lane_xor64<16>(mine) : from_lane_xor64<32>(mine);
+                    const bool keep_min = lower == ascending[t];
+                    const bool take = (other < mine) == keep_min;       // the words are never equal
+                    c[t] = take ? other : mine;
+                }
+            }
+        }
+    }
+}
+
+// bitonic_network over the first kUse of the kT slots
+template <int kUse, int kT>
+__device__ __forceinline__ void bitonic_network_of(uint64_t (&c)[kT], int lane)
+{
+    uint64_t h[kUse];
+#pragma unroll
+    for (int t = 0; t < kUse; t++) h[t] = c[t];
+    bitonic_network<kUse>(h, lane);
+#pragma unroll
+    for (int t = 0; t < kUse; t++) c[t] = h[t];
+}
+
+template <int kT>
+__device__ __forceinline__ void sort_segment_bitonic(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
+                                                     uint32_t v, int lo, int hi, uint32_t* __restrict__ seg_flags,
+                                                     uint32_t* s_v)
 {
     const int lane = threadIdx.x;
     const int len = hi - lo;
     const uint32_t upper = (uint32_t)(keys[lo] >> 32);
-    uint32_t k[kT], val[kT];
+    uint64_t c[kT];
     bool mixed = false;
 #pragma unroll
     for (int t = 0; t < kT; t++) {
         const int i = t * kWave + lane;
-        k[t] = 0xffffffffu;
-        val[t] = 0;
+        c[t] = ~0ull;
         if (i < len) {
             const uint64_t kk = keys[lo + i];
-            k[t] = (uint32_t)kk;
-            val[t] = values[lo + i];
+            c[t] = (kk << 32) | (uint32_t)i;
+            s_v[i] = values[lo + i];
             mixed = mixed || (uint32_t)(kk >> 32) != upper;
         }
     }
@@ -555,76 +633,22 @@ __device__ __forceinline__ void sort_segment_wave(uint64_t* __restrict__ keys, u
         if (seg_flags && lane == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
         return;
     }
-
-#pragma unroll 1
-    for (int shift = 0; shift < 32; shift += 8) {
-#pragma unroll
-        for (int q = 0; q < 4; q++) cnt[q * kWave + lane] = 0;
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int t = 0; t < kT; t++) {
-            if (t * kWave >= len) break;               // uniform: the remaining register slots are empty
-            if (t * kWave + lane < len) atomicAdd(&cnt[(k[t] >> shift) & 255u], 1u);
-        }
-        __builtin_amdgcn_wave_barrier();
-
-        // exclusive scan over the 256 digits; lane handles digits lane, lane+64, lane+128, lane+192
-        uint32_t base = 0;
-        bool any_full = false;
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const uint32_t c = cnt[q * kWave + lane];
-            any_full = any_full || c == (uint32_t)len;
-            uint32_t incl = wave_inclusive_sum(c);
-            cnt[q * kWave + lane] = base + incl - c;
-            base += (uint32_t)bcast_i((int)incl, kWave - 1);
-        }
-        __builtin_amdgcn_wave_barrier();
-        if (ballot(any_full)) continue;            // every pair has the same digit: nothing moves
-
-#pragma unroll
-        for (int t = 0; t < kT; t++) {
-            if (t * kWave >= len) break;
-            const bool valid = t * kWave + lane < len;
-            const uint32_t d = (k[t] >> shift) & 255u;
-            uint64_t peers = ballot(valid);
-#pragma unroll
-            for (int b = 0; b < 8; b++) {
-                const bool bit = (d >> b) & 1u;
-                const uint64_t with_bit = ballot(bit);
-                peers &= bit ? with_bit : ~with_bit;
-            }
-            const int below = popc_below(peers);
-            uint32_t before = 0;
-            if (valid && below == 0) {
-                before = cnt[d];
-                cnt[d] = before + (uint32_t)__popcll(peers);
-            }
-            const int leader = valid ? __ffsll((long long)peers) - 1 : lane;
-            before = (uint32_t)__shfl((int)before, leader);
-            if (valid) {
-                s_k[before + (uint32_t)below] = k[t];
-                s_v[before + (uint32_t)below] = val[t];
-            }
-            __builtin_amdgcn_sched_barrier(0);      // keeps the live ranges of one pair's ballots from piling up
-        }
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int t = 0; t < kT; t++) {
-            if (t * kWave >= len) break;
-            const int i = t * kWave + lane;
-            if (i < len) { k[t] = s_k[i]; val[t] = s_v[i]; }
-        }
-        __builtin_amdgcn_wave_barrier();
-    }
+    // the network over the smallest power of two of register slots that holds the segment
+    if (len <= kWave) bitonic_network_of<1>(c, lane);
+    else if (kT >= 2 && len <= 2 * kWave) bitonic_network_of<(kT >= 2 ? 2 : 1)>(c, lane);
+    else if (kT >= 4 && len <= 4 * kWave) bitonic_network_of<(kT >= 4 ? 4 : 1)>(c, lane);
+    else if (kT >= 8 && len <= 8 * kWave) bitonic_network_of<(kT >= 8 ? 8 : 1)>(c, lane);
+    else bitonic_network_of<kT>(c, lane);
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int t = 0; t < kT; t++) {
         const int i = t * kWave + lane;
         if (i < len) {
-            keys[lo + i] = ((uint64_t)upper << 32) | k[t];
-            values[lo + i] = val[t];
+            keys[lo + i] = ((uint64_t)upper << 32) | (c[t] >> 32);
+            values[lo + i] = s_v[(uint32_t)c[t]];
         }
     }
+    __builtin_amdgcn_wave_barrier();
 }
 
 // One wave per workgroup; with a table of segment starts the workgroup looks at kIds tile ids
@@ -634,35 +658,57 @@ template <int kT, int kIds>
 __global__ __launch_bounds__(kWave) void segment_sort_wave_kernel(
     uint64_t* __restrict__ keys, uint32_t* __restrict__ values, int n, uint32_t tile_mask, int min_len, uint32_t ids,
     const int* __restrict__ seg_start, uint32_t* __restrict__ seg_flags,
-    int list_min0, int list_max0, int list_max1,
-    uint32_t* __restrict__ seg_counts, uint32_t* __restrict__ list0, uint32_t* __restrict__ list1)
+    int list_max0, int list_max1, int list_max2,
+    uint32_t* __restrict__ seg_counts, uint32_t* __restrict__ list0, uint32_t* __restrict__ list1,
+    uint32_t* __restrict__ list2, uint32_t list_cap0, uint32_t list_cap1, uint32_t list_cap2)
 {
-    __shared__ uint32_t s_k[kT * kWave];
     __shared__ uint32_t s_v[kT * kWave];
-    __shared__ uint32_t s_cnt[kBins];
     const int lane = threadIdx.x;
     if (!seg_start) {
         const uint32_t v = blockIdx.x;
         const int lo = wave_lower_bound(keys, n, v, tile_mask);
         const int hi = v == tile_mask ? n : wave_lower_bound(keys, n, v + 1, tile_mask);
         if (hi - lo <= min_len || hi - lo > kT * kWave) return;
-        sort_segment_wave<kT>(keys, values, v, lo, hi, seg_flags, s_k, s_v, s_cnt);
+        sort_segment_bitonic<kT>(keys, values, v, lo, hi, seg_flags, s_v);
         return;
     }
     const uint32_t first_id = blockIdx.x * (uint32_t)kIds;
     const uint32_t mine = first_id + (uint32_t)lane;
     int len = 0;
     if (lane < kIds && mine < ids) len = seg_start[mine + 1] - seg_start[mine];
-    // This launch sees every tile id once: it also lists the ids whose segments need a multi-wave
-    // workgroup (lengths in (list_min0, list_max0] and (list_max0, list_max1]), so that those few,
-    // long-running segments can be dealt out evenly by the launches that follow.
+    // This launch sees every tile id once: it also lists the ids of the longer segments by class
+    // (lengths up to list_max0, list_max1, list_max2), so that those fewer, longer-running
+    // segments can be dealt out evenly by the launches that follow.
     if (list0) {
-        if (len > list_min0 && len <= list_max0) list0[atomicAdd(&seg_counts[0], 1u)] = mine;
-        else if (len > list_max0 && len <= list_max1) list1[atomicAdd(&seg_counts[1], 1u)] = mine;
+        const uint32_t shard = blockIdx.x % kListShards;
+        if (len > kT * kWave && len <= list_max0)
+            list0[(size_t)shard * list_cap0 + atomicAdd(&seg_counts[0 * kListShards + shard], 1u)] = mine;
+        else if (len > list_max0 && len <= list_max1)
+            list1[(size_t)shard * list_cap1 + atomicAdd(&seg_counts[1 * kListShards + shard], 1u)] = mine;
+        else if (len > list_max1 && len <= list_max2)
+            list2[(size_t)shard * list_cap2 + atomicAdd(&seg_counts[2 * kListShards + shard], 1u)] = mine;
     }
     for (uint64_t todo = ballot(len > min_len && len <= kT * kWave); todo; todo &= todo - 1) {
         const uint32_t v = first_id + (uint32_t)(__ffsll((long long)todo) - 1);
-        sort_segment_wave<kT>(keys, values, v, seg_start[v], seg_start[v + 1], seg_flags, s_k, s_v, s_cnt);
+        sort_segment_bitonic<kT>(keys, values, v, seg_start[v], seg_start[v + 1], seg_flags, s_v);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// The listed segments of one class (at most 64*kT pairs each), dealt out round-robin to
+// single-wave workgroups.
+template <int kT>
+__global__ __launch_bounds__(kWave) void segment_sort_wave_list_kernel(
+    uint64_t* __restrict__ keys, uint32_t* __restrict__ values, const int* __restrict__ seg_start,
+    uint32_t* __restrict__ seg_flags, const uint32_t* __restrict__ list, const uint32_t* __restrict__ list_count,
+    uint32_t list_cap)
+{
+    __shared__ uint32_t s_v[kT * kWave];
+    const uint32_t shard = blockIdx.x % kListShards;
+    const uint32_t count = list_count[shard];
+    for (uint32_t i = blockIdx.x / kListShards; i < count; i += gridDim.x / kListShards) {
+        const uint32_t v = list[(size_t)shard * list_cap + i];
+        sort_segment_bitonic<kT>(keys, values, v, seg_start[v], seg_start[v + 1], seg_flags, s_v);
         __builtin_amdgcn_wave_barrier();
     }
 }
@@ -751,7 +797,7 @@ __global__ __launch_bounds__(kSortBlock) void segment_sort_general_kernel(
     }
 }
 
-constexpr int kCapTiny = 256, kCapSmall = 1024, kCapMedium = 4096, kCapLarge = 8192;
+constexpr int kCapTiny = 512, kCapSmall = 1024, kCapMedium = 4096, kCapLarge = 8192;
 
 
 } // namespace
@@ -838,29 +884,44 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         uint64_t* ks = gaussian_keys_sorted;
         uint32_t* vs = gaussian_values_sorted;
         uint32_t* seg_counts = (uint32_t*)(list_sorting_space + ws.seg_lists);
-        uint32_t* list_medium = seg_counts + 64;
-        uint32_t* list_large = list_medium + ((size_t)n / 1024 + 2);
+        const uint32_t cap_small = (uint32_t)(n / 512 + 2), cap_medium = (uint32_t)(n / 1024 + 2), cap_large = (uint32_t)(n / 4096 + 2);
+        uint32_t* list_small = seg_counts + 128;
+        uint32_t* list_medium = list_small + (size_t)kListShards * cap_small;
+        uint32_t* list_large = list_medium + (size_t)kListShards * cap_medium;
         const uint32_t* no_list = nullptr;
-#define FGS_SEGMENT_CLASS(WAVES, CAP, IDS, MINLEN, GRID, LIST, COUNT)                                         \
+        // grids of the list-driven launches: a multiple of kListShards, enough for every listed segment
+        auto list_grid = [](unsigned most, unsigned limit) {
+            const unsigned g = most < limit ? most : limit;
+            return (g + kListShards - 1) / kListShards * kListShards;
+        };
+#define FGS_SEGMENT_CLASS(WAVES, CAP, IDS, MINLEN, GRID, LIST, COUNT, LISTCAP)                                \
         hipLaunchKernelGGL((segment_sort_kernel<WAVES, CAP, IDS>), dim3(GRID), dim3((WAVES) * kWave), 0, st,  \
                            ks, vs, n, tile_mask, MINLEN, ids, (const int*)seg_start, seg_flags,               \
-                           (const uint32_t*)(LIST), (const uint32_t*)(COUNT))
-        // one or two tile ids per wave: neighbouring tiles tend to be equally busy, so a wave that
-        // took several of them would become the tail of the launch
+                           (const uint32_t*)(LIST), (const uint32_t*)(COUNT), LISTCAP)
+        // Up to 512 pairs: one wave, bitonic network in registers; one or two tile ids per wave
+        // (neighbouring tiles tend to be equally busy, so a wave that took several of them would
+        // become the tail of the launch).  With a table the launch also lists the longer segments.
         hipLaunchKernelGGL((segment_sort_wave_kernel<kCapTiny / kWave, 2>), dim3(seg_start ? (ids + 1) / 2 : ids), dim3(kWave),
                            0, st, ks, vs, n, tile_mask, 1, ids, (const int*)seg_start, seg_flags,
-                           kCapSmall, kCapMedium, kCapLarge, seg_counts, seg_start ? list_medium : nullptr, list_large);
-        if (n > kCapTiny) FGS_SEGMENT_CLASS(4, kCapSmall, 1, kCapTiny, ids, no_list, no_list);
+                           kCapSmall, kCapMedium, kCapLarge, seg_counts, seg_start ? list_small : nullptr, list_medium,
+                           list_large, cap_small, cap_medium, cap_large);
         if (seg_start) {
+            if (n > kCapTiny)       // 513..1024: the same network over 16 register slots, from the lists
+                hipLaunchKernelGGL((segment_sort_wave_list_kernel<kCapSmall / kWave>),
+                                   dim3(list_grid((unsigned)(n / (kCapTiny + 1) + 1), 8192u)),
+                                   dim3(kWave), 0, st, ks, vs, (const int*)seg_start, seg_flags,
+                                   (const uint32_t*)list_small, (const uint32_t*)seg_counts, cap_small);
             if (n > kCapSmall) {
-                const unsigned most_m = (unsigned)(n / (kCapSmall + 1) + 1), most_l = (unsigned)(n / (kCapMedium + 1) + 1);
-                FGS_SEGMENT_CLASS(8, kCapMedium, 64, kCapSmall, most_m < 1024u ? most_m : 1024u, list_medium, seg_counts);
+                FGS_SEGMENT_CLASS(8, kCapMedium, 64, kCapSmall, list_grid((unsigned)(n / (kCapSmall + 1) + 1), 1024u),
+                                  list_medium, seg_counts + kListShards, cap_medium);
                 if (n > kCapMedium)
-                    FGS_SEGMENT_CLASS(16, kCapLarge, 64, kCapMedium, most_l < 256u ? most_l : 256u, list_large, seg_counts + 1);
+                    FGS_SEGMENT_CLASS(16, kCapLarge, 64, kCapMedium, list_grid((unsigned)(n / (kCapMedium + 1) + 1), 256u),
+                                      list_large, seg_counts + 2 * kListShards, cap_large);
             }
         } else {
-            if (n > kCapSmall) FGS_SEGMENT_CLASS(8, kCapMedium, 64, kCapSmall, ids, no_list, no_list);
-            if (n > kCapMedium) FGS_SEGMENT_CLASS(16, kCapLarge, 64, kCapMedium, ids, no_list, no_list);
+            if (n > kCapTiny) FGS_SEGMENT_CLASS(4, kCapSmall, 1, kCapTiny, ids, no_list, no_list, 0u);
+            if (n > kCapSmall) FGS_SEGMENT_CLASS(8, kCapMedium, 64, kCapSmall, ids, no_list, no_list, 0u);
+            if (n > kCapMedium) FGS_SEGMENT_CLASS(16, kCapLarge, 64, kCapMedium, ids, no_list, no_list, 0u);
         }
 #undef FGS_SEGMENT_CLASS
         hipLaunchKernelGGL(segment_sort_general_kernel, dim3(seg_start ? (ids + kWave - 1) / kWave : ids),
