@@ -8,16 +8,19 @@
 //
 //  1. Partition by tile id: one stable counting pass per 8 bits of tile id (two passes for up to
 //     65536 tiles).  A pass is count -> offsets -> scatter: `count_kernel` builds one digit
-//     histogram per block of 2048 pairs, `chunk_sum_kernel` + `offsets_kernel` turn the
+//     histogram per block of 4096 pairs, `chunk_sum_kernel` + `offsets_kernel` turn the
 //     histograms into the exclusive start of every (block, digit) run, and `scatter_kernel` ranks
 //     its block in LDS (wave64 ballot matching, so equal digits keep their input order) and
 //     writes each run to its start.  No workgroup ever waits for another one.
-//  2. Sort every tile's segment by the 32 depth bits, in LDS: `segment_starts_kernel` tabulates
-//     where each tile id's segment begins; a `segment_sort_kernel` workgroup loads a segment, runs up to four stable 8-bit counting passes without touching memory (a pass in
-//     which all pairs share the digit is skipped) and writes the segment back in place.  Segments
-//     are handled by size class - one wave up to 256 and up to 1024 pairs, four waves up to
-//     4096, sixteen waves up to 8192; longer ones, and segments whose keys differ above the sorted bit range,
-//     go through the same passes with the ping-pong copy in HBM instead of LDS.
+//  2. Sort every tile's segment by the 32 depth bits without touching memory in between:
+//     `segment_starts_kernel` tabulates where each tile id's segment begins, then segments are
+//     handled by size class.  Up to 1024 pairs one wave holds the segment in registers as 64-bit
+//     words depth << 32 | position and runs a bitonic network on them (all words differ, so the
+//     result is that of a stable sort by depth); lane exchanges inside a row of 16 lanes are
+//     data-parallel-primitive moves.  Up to 4096 (8 waves) and 8192 pairs (16 waves) a workgroup
+//     runs up to four stable 8-bit counting passes in LDS, skipping a pass in which all pairs
+//     share the digit.  Longer segments, and segments whose keys differ above the sorted bit
+//     range, go through the same passes with the ping-pong copy in HBM instead of LDS.
 //
 // Bytes moved per pair: 8 (count) + 24 (scatter) per partition pass, 24 for the segment sort:
 // 88 for two partition passes, against 8 + 6 * 24 = 152 for a six-pass LSD sort of 47 bits.
