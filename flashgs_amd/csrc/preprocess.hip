@@ -28,6 +28,7 @@ constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kStashCap = 1024;         // flat candidates (and so stashed hits) per wave
 constexpr int kHugeMin = 1024;          // rectangles with more tiles than this are tested by the whole workgroup
 constexpr int kHugeCap = 16;            // such rectangles per workgroup; further ones stay with their wave
+constexpr int kSpanWords = kWavesPerBlock * kStashCap / 4;   // column + row spans of one listed rectangle
 constexpr unsigned kSpinLimit = 1u << 22;   // polls before a chained-scan wait gives up
 
 struct Camera {
@@ -134,13 +135,41 @@ __device__ __forceinline__ void cov2d(const float t_in[3], const Camera& cam, co
     c11 = cov.c[1][1] + 0.3f;
 }
 
-// preprocess.cu:187-194
-__device__ __forceinline__ bool segment_hits(float a, float b, float c, float d, float l, float r)
+// The ellipse/tile test of the reference (preprocess.cu:187-241), cut into the pieces that depend
+// on one tile coordinate only.  For the test against the nearer vertical edge of tile column x
+// (preprocess.cu:196-215 with the segment test :187-194): a = conic z, b = -2 conic_y dx,
+// c = conic_x dx^2 - w, delta = b^2 - 4ac depend on x alone, and tile row y enters through
+//   t1 = (top - cy) 2a + b,     near_ok = t1 <= 0 || t1^2 <= delta,
+//   t2 = (bottom - cy) 2a + b,  far_ok  = t2 >= 0 || t2^2 <= delta.
+// The test against the nearer horizontal edge is the same with the axes exchanged.  Every
+// expression is evaluated exactly as the reference writes it, one IEEE operation at a time.
+struct EdgeTest {
+    float two_a, b, delta;
+};
+
+// centre: the Gaussian's coordinate across the edge; lo, hi: first and last pixel of the tile
+// across the edge; a: conic entry along the edge, c_across: conic entry across it
+__device__ __forceinline__ EdgeTest edge_test(float a, float cony, float c_across, float centre, int lo, int hi, float w)
 {
-    float delta = b * b - 4.0f * a * c;
-    float t1 = (l - d) * (2.0f * a) + b;
-    float t2 = (r - d) * (2.0f * a) + b;
-    return delta >= 0.0f && (t1 <= 0.0f || t1 * t1 <= delta) && (t2 >= 0.0f || t2 * t2 <= delta);
+    const float d = (centre * 2.0f < (float)(lo + hi)) ? centre - (float)lo : centre - (float)hi;
+    EdgeTest e;
+    e.b = -2.0f * cony * d;
+    const float c = c_across * d * d - w;
+    e.delta = e.b * e.b - 4.0f * a * c;
+    e.two_a = 2.0f * a;
+    return e;
+}
+
+__device__ __forceinline__ bool near_ok(const EdgeTest& e, float first_px, float centre_along)
+{
+    const float t1 = (first_px - centre_along) * e.two_a + e.b;
+    return t1 <= 0.0f || t1 * t1 <= e.delta;
+}
+
+__device__ __forceinline__ bool far_ok(const EdgeTest& e, float last_px, float centre_along)
+{
+    const float t2 = (last_px - centre_along) * e.two_a + e.b;
+    return t2 >= 0.0f || t2 * t2 <= e.delta;
 }
 
 // preprocess.cu:238-241 || :196-236 for tile (x, y)
@@ -153,17 +182,41 @@ __device__ __forceinline__ bool tile_hit(int x, int y, int bx, int by, float cx,
     if (cx >= fminx && cx <= fmaxx && cy >= fminy && cy <= fmaxy) return true;
 
     const float w = 2.0f * power;
-    float dx = (cx * 2.0f < (float)(minx + maxx)) ? cx - fminx : cx - fmaxx;
-    float a = conz;
-    float b = -2.0f * cony * dx;
-    float c = conx * dx * dx - w;
-    if (segment_hits(a, b, c, cy, fminy, fmaxy)) return true;
+    const EdgeTest v = edge_test(conz, cony, conx, cx, minx, maxx, w);
+    if (v.delta >= 0.0f && near_ok(v, fminy, cy) && far_ok(v, fmaxy, cy)) return true;
+    const EdgeTest h = edge_test(conx, cony, conz, cy, miny, maxy, w);
+    return h.delta >= 0.0f && near_ok(h, fminx, cx) && far_ok(h, fmaxx, cx);
+}
 
-    float dy = (cy * 2.0f < (float)(miny + maxy)) ? cy - fminy : cy - fmaxy;
-    a = conx;
-    b = -2.0f * cony * dy;
-    c = conz * dy * dy - w;
-    return segment_hits(a, b, c, cx, fminx, fmaxx);
+// For one tile column (or row) of a rectangle: which of the `count` tiles along it pass the edge
+// test.  near_ok can only turn from true to false and far_ok from false to true as the tile index
+// grows (both t1 and t2 are non-decreasing in it when 2a > 0: every operation that leads to them
+// is monotone, rounding included), so the tiles that pass are the interval between two points
+// that bisection finds with the very predicates of the per-tile test.  Packed as
+// first | last << 15 | centre-inside-this-column << 30; an empty interval is first 1, last 0.
+__device__ __forceinline__ uint32_t edge_span(float a, float cony, float c_across, float centre, float centre_along,
+                                              int tile, int block, int first_tile_along, int block_along, int count, float w)
+{
+    const int lo_px = tile * block, hi_px = lo_px + block - 1;
+    const uint32_t inside = (centre >= (float)lo_px && centre <= (float)hi_px) ? 1u << 30 : 0u;
+    const EdgeTest e = edge_test(a, cony, c_across, centre, lo_px, hi_px, w);
+    if (!(e.delta >= 0.0f)) return inside | 1u;
+    int lo = 0, hi = count;             // near_ok holds for tiles [0, lo), fails from hi on
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (near_ok(e, (float)((first_tile_along + mid) * block_along), centre_along)) lo = mid + 1;
+        else hi = mid;
+    }
+    const int last = lo - 1;
+    lo = 0; hi = count;                 // far_ok fails for tiles [0, lo), holds from hi on
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (far_ok(e, (float)((first_tile_along + mid) * block_along + block_along - 1), centre_along)) hi = mid;
+        else lo = mid + 1;
+    }
+    const int first = lo;
+    if (first > last) return inside | 1u;
+    return inside | (uint32_t)first | ((uint32_t)last << 15);
 }
 
 // j / w and j % w for 0 <= j, 1 <= w.  Below 2^20 the quotient comes from a reciprocal estimate
@@ -351,12 +404,15 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     __shared__ uint32_t s_block_base;
     __shared__ uint32_t s_stash[kWavesPerBlock][kStashCap];     // hits of the flat candidates, in emission order
     __shared__ uint64_t s_hits[kWavesPerBlock][kStashCap / kWave + 1];
-    __shared__ uint8_t s_owner[kWavesPerBlock][kStashCap];      // flat candidate -> lane that owns it
+    // flat candidate -> lane that owns it; free again after the flat tile tests, when the listed
+    // rectangles use it for their column and row spans
+    __shared__ __align__(4) uint8_t s_owner[kWavesPerBlock][kStashCap];
     // rectangles too big for one wave: parameters, per-wave hit counts, first key slot
     __shared__ float s_huge_f[kHugeCap][6];
     __shared__ int s_huge_i[kHugeCap][4];
     __shared__ uint32_t s_huge_u[kHugeCap][3];                  // depth bits, Gaussian index, first slot
     __shared__ uint32_t s_huge_cnt[kHugeCap][kWavesPerBlock];
+    __shared__ int s_huge_spans[kHugeCap];                      // 1: the tiles that pass are found from column and row spans
     __shared__ int s_nhuge;
 
     const int tid = threadIdx.x;
@@ -468,6 +524,13 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
             s_huge_f[e][3] = cony; s_huge_f[e][4] = conz; s_huge_f[e][5] = power;
             s_huge_i[e][0] = rminx; s_huge_i[e][1] = rminy; s_huge_i[e][2] = rw; s_huge_i[e][3] = area;
             s_huge_u[e][0] = __float_as_uint(depth); s_huge_u[e][1] = (uint32_t)idx;
+            // Spans need 2a > 0 for both edge directions and values that cannot overflow on the
+            // way to t1, t2 (the monotonicity argument assumes no NaN), and room for one word
+            // per column and row; everything else is tested tile by tile.
+            const float big = 1e30f;
+            s_huge_spans[e] = conx > 0.0f && conz > 0.0f && conx < big && conz < big && fabsf(cony) < big &&
+                              fabsf(cx) < 1e9f && fabsf(cy) < 1e9f && fabsf(power) < big &&
+                              rw + rh <= kSpanWords;
         }
     }
     const bool large = has_tiles && !flat && huge_slot < 0;
@@ -542,10 +605,37 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     // the listed rectangles: wave w counts tiles [w*part, (w+1)*part) of each
     __syncthreads();
     const int n_huge = min(s_nhuge, kHugeCap);
-    for (int e = 0; e < n_huge; e++) {
+    uint32_t* const spans = reinterpret_cast<uint32_t*>(&s_owner[0][0]);
+    // Fills spans[0, rw) with the rows that pass the vertical-edge test in each column of the
+    // rectangle and spans[rw, rw + rh) with the columns that pass the horizontal-edge test in
+    // each row.  All threads of the workgroup call it; barriers before and after.
+    auto fill_spans = [&](int e) {
         const float gcx = s_huge_f[e][0], gcy = s_huge_f[e][1];
-        const float gconx = s_huge_f[e][2], gcony = s_huge_f[e][3], gconz = s_huge_f[e][4], gpower = s_huge_f[e][5];
-        const int gminx = s_huge_i[e][0], gminy = s_huge_i[e][1], grw = s_huge_i[e][2], garea = s_huge_i[e][3];
+        const float gconx = s_huge_f[e][2], gcony = s_huge_f[e][3], gconz = s_huge_f[e][4];
+        const float w = 2.0f * s_huge_f[e][5];
+        const int gminx = s_huge_i[e][0], gminy = s_huge_i[e][1], grw = s_huge_i[e][2];
+        const int grh = s_huge_i[e][3] / grw;
+        __syncthreads();
+        for (int i = tid; i < grw + grh; i += kBlock)
+            spans[i] = i < grw ? edge_span(gconz, gcony, gconx, gcx, gcy, gminx + i, cam.bx, gminy, cam.by, grh, w)
+                               : edge_span(gconx, gcony, gconz, gcy, gcx, gminy + i - grw, cam.by, gminx, cam.bx, grw, w);
+        __syncthreads();
+    };
+    // whether tile (tx, ty) of rectangle e passes: from the spans, or by the full test
+    auto listed_tile_hit = [&](int e, bool from_spans, int tx, int ty, int grw) {
+        if (from_spans) {
+            const uint32_t col = spans[tx], row = spans[grw + ty];
+            const bool by_column = (uint32_t)ty >= (col & 0x7fffu) && (uint32_t)ty <= ((col >> 15) & 0x7fffu);
+            const bool by_row = (uint32_t)tx >= (row & 0x7fffu) && (uint32_t)tx <= ((row >> 15) & 0x7fffu);
+            return by_column || by_row || ((col & row) >> 30) != 0;
+        }
+        return tile_hit(s_huge_i[e][0] + tx, s_huge_i[e][1] + ty, cam.bx, cam.by, s_huge_f[e][0], s_huge_f[e][1],
+                        s_huge_f[e][2], s_huge_f[e][3], s_huge_f[e][4], s_huge_f[e][5]);
+    };
+    for (int e = 0; e < n_huge; e++) {
+        const bool from_spans = s_huge_spans[e] != 0;
+        if (from_spans) fill_spans(e);
+        const int grw = s_huge_i[e][2], garea = s_huge_i[e][3];
         const int part = ((garea + kWavesPerBlock - 1) / kWavesPerBlock + kWave - 1) / kWave * kWave;
         const int j_lo = min(garea, wave * part), j_hi = min(garea, j_lo + part);
         uint32_t total = 0;
@@ -555,7 +645,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
             if (j < j_hi) {
                 int tx, ty;
                 div_mod(j, grw, ty, tx);
-                ok = tile_hit(gminx + tx, gminy + ty, cam.bx, cam.by, gcx, gcy, gconx, gcony, gconz, gpower);
+                ok = listed_tile_hit(e, from_spans, tx, ty, grw);
             }
             total += (uint32_t)__popcll(ballot(ok));
         }
@@ -624,8 +714,8 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         if (huge_slot >= 0) s_huge_u[huge_slot][2] = my_slot;
         __syncthreads();
         for (int e = 0; e < n_huge; e++) {
-            const float gcx = s_huge_f[e][0], gcy = s_huge_f[e][1];
-            const float gconx = s_huge_f[e][2], gcony = s_huge_f[e][3], gconz = s_huge_f[e][4], gpower = s_huge_f[e][5];
+            const bool from_spans = s_huge_spans[e] != 0;
+            if (from_spans) fill_spans(e);
             const int gminx = s_huge_i[e][0], gminy = s_huge_i[e][1], grw = s_huge_i[e][2], garea = s_huge_i[e][3];
             const uint32_t gdepth = s_huge_u[e][0], gidx = s_huge_u[e][1];
             uint64_t slot = s_huge_u[e][2];
@@ -639,7 +729,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
                 int tx = 0, ty = 0;
                 if (j < j_hi) {
                     div_mod(j, grw, ty, tx);
-                    ok = tile_hit(gminx + tx, gminy + ty, cam.bx, cam.by, gcx, gcy, gconx, gcony, gconz, gpower);
+                    ok = listed_tile_hit(e, from_spans, tx, ty, grw);
                 }
                 const uint64_t hits = ballot(ok);
                 if (ok) {
