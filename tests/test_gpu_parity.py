@@ -416,6 +416,23 @@ def test_sort_segment_size_classes(seg):
     _sort_case(tile, depth.view(np.uint32), W, H, seed=seg)
 
 
+def test_sort_every_segment_length_up_to_1100():
+    """One tile per length 1 ... 1100: every padding of the register sorting networks (64, 128, ... 1024
+    elements) and the first lengths of the next class, with many equal depths (ties must keep input
+    order) and with depths of all magnitudes, 0 and 0xffffffff included."""
+    rng = np.random.default_rng(1100)
+    W, H = 1920, 1080
+    lengths = np.arange(1, 1101)
+    tiles = rng.permutation(120 * 68)[:lengths.size].astype(np.uint32)
+    tile = np.repeat(tiles, lengths)
+    depth = rng.integers(0, 1 << 32, tile.size, dtype=np.uint64).astype(np.uint32)
+    depth[::5] = depth[1::5][: depth[::5].size]          # duplicates next to each other before the shuffle
+    depth[rng.integers(0, tile.size, 2000)] = 0
+    depth[rng.integers(0, tile.size, 2000)] = 0xFFFFFFFF
+    order = rng.permutation(tile.size)
+    _sort_case(tile[order], depth[order], W, H, seed=7)
+
+
 def test_sort_bits_above_the_range_stay_with_their_pair():
     """Bits above 32 + bit_length(tiles) are outside the sorted range (sort.cu:34-39) but travel
     with the key; segments whose keys differ there take the general path."""
