@@ -25,7 +25,7 @@ extern "C" {
 #define FGS_E_HIP        -3   /* a HIP runtime call or kernel launch failed */
 #define FGS_E_NOMEM      -4   /* internal scratch allocation failed */
 
-/* Largest key count the sort accepts (status words carry 30-bit counts). */
+/* Largest key count the sort accepts (positions and block counts are kept in 32-bit integers). */
 #define FGS_MAX_RENDERED ((1 << 30) - 1)
 
 /*
@@ -45,6 +45,13 @@ extern "C" {
  * value buffers hold.  Pairs that would land at or beyond it are dropped (the counter still
  * counts them, so the caller's check of example.py:79-82 keeps working); pass 0 to write
  * unchecked like the reference (preprocess.cu:330,395).
+ *
+ * The call is asynchronous on `stream`.  The library keeps a small per-device scratch for the
+ * scan over workgroups (allocated on first use, grown when a larger P arrives - the only times
+ * the call synchronises); calls on one device must not overlap in time.  Nothing on the host
+ * changes from launch to launch, so once the scratch is large enough a launch can be captured in
+ * a HIP graph and replayed.  If the scan ever times out waiting for a workgroup, *curr_offset is
+ * set to INT_MIN.
  */
 int fgs_preprocess(int P,
                    const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
