@@ -683,7 +683,8 @@ __global__ __launch_bounds__(kWave) void segment_sort_wave_kernel(
     // (lengths up to list_max0, list_max1, list_max2), so that those fewer, longer-running
     // segments can be dealt out evenly by the launches that follow.
     if (list0) {
-        const uint32_t shard = blockIdx.x % kListShards;
+        // neighbouring tiles tend to be equally busy: mix the index so that every list gets its share
+        const uint32_t shard = (blockIdx.x ^ (blockIdx.x >> 5) ^ (blockIdx.x >> 10) ^ (blockIdx.x >> 15)) % kListShards;
         if (len > kT * kWave && len <= list_max0)
             list0[(size_t)shard * list_cap0 + atomicAdd(&seg_counts[0 * kListShards + shard], 1u)] = mine;
         else if (len > list_max0 && len <= list_max1)
@@ -901,10 +902,10 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         hipLaunchKernelGGL((segment_sort_kernel<WAVES, CAP, IDS>), dim3(GRID), dim3((WAVES) * kWave), 0, st,  \
                            ks, vs, n, tile_mask, MINLEN, ids, (const int*)seg_start, seg_flags,               \
                            (const uint32_t*)(LIST), (const uint32_t*)(COUNT), LISTCAP)
-        // Up to 512 pairs: one wave, bitonic network in registers; one or two tile ids per wave
-        // (neighbouring tiles tend to be equally busy, so a wave that took several of them would
-        // become the tail of the launch).  With a table the launch also lists the longer segments.
-        hipLaunchKernelGGL((segment_sort_wave_kernel<kCapTiny / kWave, 2>), dim3(seg_start ? (ids + 1) / 2 : ids), dim3(kWave),
+        // Up to 512 pairs: one wave, bitonic network in registers; one tile id per wave (neighbouring
+        // tiles tend to be equally busy, so a wave that took several of them would become the tail
+        // of the launch).  With a table the launch also lists the longer segments.
+        hipLaunchKernelGGL((segment_sort_wave_kernel<kCapTiny / kWave, 1>), dim3(ids), dim3(kWave),
                            0, st, ks, vs, n, tile_mask, 1, ids, (const int*)seg_start, seg_flags,
                            kCapSmall, kCapMedium, kCapLarge, seg_counts, seg_start ? list_small : nullptr, list_medium,
                            list_large, cap_small, cap_medium, cap_large);
