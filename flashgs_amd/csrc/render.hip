@@ -153,6 +153,12 @@ __device__ __forceinline__ void blend_tile(
     if (tile_x >= tiles_x || tile_y >= tiles_y) return;
     const int2 range = ranges[tile_y * tiles_x + tile_x];
     const int n = range.y - range.x;
+    // A launch ends when its longest list ends, and a wave that shares its SIMD equally with the
+    // waves of short lists gets to its own end late: waves with long lists ask for a higher
+    // issue priority.
+    if (n > 1024) __builtin_amdgcn_s_setprio(3);
+    else if (n > 512) __builtin_amdgcn_s_setprio(2);
+    else if (n > 256) __builtin_amdgcn_s_setprio(1);
 
     // lane -> 2x2 quad of every 16x16 sub-tile
     const int qx = (lane & 7) * 2, qy = (lane >> 3) * 2;
