@@ -332,6 +332,42 @@ def test_sort_sizes_against_numpy(n):
     assert np.array_equal(gp.u32(vs)[:n], vals[order])
 
 
+def test_sort_8k_frame_three_partition_passes():
+    """7680x4320 has 129 600 tiles: 17 tile bits, three partition passes.  Against numpy."""
+    rng = np.random.default_rng(8)
+    n = 1_200_000
+    tile = rng.integers(0, 480 * 270, n).astype(np.uint32)
+    tile[: n // 6] = 129_599                      # one very long segment in the last tile
+    depth = rng.uniform(0.2, 90.0, n).astype(np.float32)
+    depth[::7] = np.float32(3.25)
+    _sort_case(tile, depth.view(np.uint32), 7680, 4320, seed=8)
+
+
+def test_sort_120M_pairs_properties():
+    """120M pairs on an 8K frame (the size the large-scale configuration speaks of), without the
+    oracle: output non-decreasing, pairs stay together, equal keys keep their input order, and
+    the output is a permutation of the input."""
+    import gpu_pipeline as gp
+    import torch
+    n = 120_000_000
+    g = torch.Generator(device=gp.DEV).manual_seed(3)
+    tile = torch.randint(0, 480 * 270, (n,), device=gp.DEV, generator=g, dtype=torch.int64)
+    depth = (torch.rand(n, device=gp.DEV, generator=g) * 90 + 0.2).to(torch.float32).view(torch.int32).to(torch.int64)
+    depth[: n // 8] = depth[0]
+    keys = (tile << 32) | depth
+    del tile, depth
+    vals = torch.arange(n, device=gp.DEV, dtype=torch.int32)        # value = input position
+    ks, vs = gp.sort(n, 7680, 4320, keys, vals)
+    assert bool((ks[1:] >= ks[:-1]).all())
+    assert bool((keys[vs.long()] == ks).all())                        # pairs stayed together
+    tie = ks[1:] == ks[:-1]
+    assert bool((vs[1:][tie] > vs[:-1][tie]).all())                   # stable
+    del tie
+    seen = torch.zeros(n, device=gp.DEV, dtype=torch.bool)
+    seen[vs.long()] = True
+    assert bool(seen.all())                                           # a permutation
+
+
 def test_sort_full_size_properties():
     """At the headline size (8M pairs, 47 key bits) without the oracle: output is a permutation of
     the input, non-decreasing, and equal keys keep their input order."""
