@@ -11,7 +11,9 @@
 //    ascending Gaussian index, then row-major tiles.  A stable sort then fixes tie order too.
 //  * The candidate tiles of all Gaussians of a wave with rectangles of at most 64 tiles are laid
 //    end to end and tested one per lane per step, so lanes stay busy whatever the mix of sizes;
-//    larger rectangles are tested by the whole wave, 64 tiles a step.
+//    larger rectangles are tested by the whole wave, 64 tiles a step, and rectangles of more than
+//    1024 tiles by the whole workgroup, which gets the passing tiles of every column and row as
+//    an interval found by bisection with the reference's own edge predicates.
 //
 // THIS FILE MUST BE COMPILED WITH -ffp-contract=off.  Every fp32 expression that feeds a key is
 // written in the operand order of the reference and has to be evaluated one IEEE operation at a
