@@ -45,7 +45,48 @@ def parse():
     ap.add_argument("--cpu-reps", type=int, default=3)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy, as the known-size reference for FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also measure what this GPU attains on a stream copy, a stream read and fp32 FMA / exp2 issue "
+                         "(libflashgs_calibrate.so) and report it under \"calibration\"")
     return ap.parse_args()
+
+
+def calibrate(torch, dev):
+    """Attained rates of this GPU on the resources the rooflines are priced against."""
+    import ctypes as C
+    from flashgs_amd import build
+    if not os.path.exists(build.CAL_PATH):
+        raise ImportError("%s is missing: run `python -m flashgs_amd.build` first" % build.CAL_PATH)
+    lib = C.CDLL(build.CAL_PATH)
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    nbytes = 1 << 30
+    src = torch.ones(nbytes // 4, device=dev, dtype=torch.float32)
+    dst = torch.empty_like(src)
+    sink = torch.zeros(4, device=dev, dtype=torch.float32)
+    out = C.c_double(0.0)
+
+    def call(fn, *a):
+        rc = fn(*a, C.byref(out), st)
+        if rc != 0:
+            raise RuntimeError("calibration kernel failed: HIP error %d" % rc)
+        return out.value
+
+    copy = call(lib.fgs_cal_copy, C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), C.c_size_t(nbytes))
+    read = call(lib.fgs_cal_read, C.c_void_p(src.data_ptr()), C.c_void_p(sink.data_ptr()), C.c_size_t(nbytes))
+    fma = call(lib.fgs_cal_alu, C.c_int(0), C.c_void_p(sink.data_ptr()))
+    mix4 = call(lib.fgs_cal_alu, C.c_int(1), C.c_void_p(sink.data_ptr()))
+    mix8 = call(lib.fgs_cal_alu, C.c_int(2), C.c_void_p(sink.data_ptr()))
+    exp = call(lib.fgs_cal_alu, C.c_int(3), C.c_void_p(sink.data_ptr()))
+    torch.cuda.synchronize()
+    return {
+        "copy_GBs_read_plus_write": round(copy / 1e9, 1), "read_GBs": round(read / 1e9, 1),
+        "fma_T_lane_ops_per_s": round(fma / 1e12, 2), "fma_TFLOPs": round(2 * fma / 1e12, 2),
+        "exp2_plus_sub_T_lane_ops_per_s": round(exp / 1e12, 2),
+        "fma_and_exp2_4to1_T_lane_ops_per_s": round(mix4 / 1e12, 2),
+        "fma_and_exp2_8to1_T_lane_ops_per_s": round(mix8 / 1e12, 2),
+        "note": "1 GiB buffers; lane-ops = wave64 instructions x 64; packed fp32 is switched off, so the FMA figure "
+                "is the non-packed issue rate (the published 157.3 TFLOP/s counts packed FMA)",
+    }
 
 
 def cpu_baseline(sc, cam, capacity, reps):
@@ -236,6 +277,8 @@ def main():
         frame_ms.sort()
         result["frame_ms_p50"] = round(frame_ms[len(frame_ms) // 2], 4)
         result["frame_ms_p99"] = round(frame_ms[min(len(frame_ms) - 1, int(0.99 * len(frame_ms)))], 4)
+    if args.calibrate:
+        result["calibration"] = calibrate(torch, dev)
     print(json.dumps(result))
 
 

@@ -18,6 +18,7 @@ CSRC = os.path.join(PKG, "csrc")
 LIB_DIR = os.path.join(PKG, "lib")
 OBJ_DIR = os.path.join(LIB_DIR, "obj")
 LIB_PATH = os.path.join(LIB_DIR, "libflashgs_hip.so")
+CAL_PATH = os.path.join(LIB_DIR, "libflashgs_calibrate.so")     # microbenchmarks for bench.py --calibrate
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
@@ -47,6 +48,7 @@ def build_lib():
         _run([HIPCC] + HIP_FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj])
         objs.append(obj)
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs)
+    _run([HIPCC] + HIP_FLAGS + ["-shared", os.path.join(CSRC, "calibrate.hip"), "-o", CAL_PATH])
     return LIB_PATH
 
 
