@@ -45,6 +45,8 @@ def parse():
     ap.add_argument("--cpu-reps", type=int, default=3)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy, as the known-size reference for FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--size", default=None, metavar="WxH",
+                    help="frame size for the trajectory workload (config 4), e.g. 3840x2160; default 1920x1080")
     ap.add_argument("--calibrate", action="store_true",
                     help="also measure what this GPU attains on a stream copy, a stream read and fp32 FMA / exp2 issue "
                          "(libflashgs_calibrate.so) and report it under \"calibration\"")
@@ -136,7 +138,12 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
 
-    sc = scenes.make(args.config)
+    kw = {}
+    if args.size:
+        if args.config != 4:
+            sys.exit("bench.py: --size applies to the trajectory workload (--config 4) only")
+        kw["width"], kw["height"] = (int(v) for v in args.size.lower().split("x"))
+    sc = scenes.make(args.config, **kw)
     cams = sc.cameras
     cam = cams[0]
     W, H = cam.width, cam.height

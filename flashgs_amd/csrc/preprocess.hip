@@ -414,6 +414,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     __shared__ int s_huge_i[kHugeCap][4];
     __shared__ uint32_t s_huge_u[kHugeCap][3];                  // depth bits, Gaussian index, first slot
     __shared__ uint32_t s_huge_cnt[kHugeCap][kWavesPerBlock];
+    __shared__ uint32_t s_chunk_rows[kWavesPerBlock][kSpanWords / kWave];   // rows covered by the column spans of 64 columns
     __shared__ int s_huge_spans[kHugeCap];                      // 1: the tiles that pass are found from column and row spans
     __shared__ int s_nhuge;
 
@@ -623,34 +624,73 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
                                : edge_span(gconx, gcony, gconz, gcy, gcx, gminy + i - grw, cam.by, gminx, cam.bx, grw, w);
         __syncthreads();
     };
-    // whether tile (tx, ty) of rectangle e passes: from the spans, or by the full test
-    auto listed_tile_hit = [&](int e, bool from_spans, int tx, int ty, int grw) {
+    // Walks the tiles of listed rectangle e that are this wave's share, in row-major order, and
+    // calls visit(tx, ty, passes) once per step of 64 tiles with every lane's own tile.
+    //  * With spans the share is a quarter of the rows.  A step covers 64 columns of one row;
+    //    it is skipped when neither the column spans of those columns reach the row (their
+    //    union is kept per 64 columns) nor the row's own span reaches the columns.
+    //  * Without spans the share is a quarter of the tiles, each tested in full.
+    auto walk_listed = [&](int e, bool from_spans, auto&& visit) {
+        const int gminx = s_huge_i[e][0], gminy = s_huge_i[e][1], grw = s_huge_i[e][2], garea = s_huge_i[e][3];
         if (from_spans) {
-            const uint32_t col = spans[tx], row = spans[grw + ty];
-            const bool by_column = (uint32_t)ty >= (col & 0x7fffu) && (uint32_t)ty <= ((col >> 15) & 0x7fffu);
-            const bool by_row = (uint32_t)tx >= (row & 0x7fffu) && (uint32_t)tx <= ((row >> 15) & 0x7fffu);
-            return by_column || by_row || ((col & row) >> 30) != 0;
+            const int grh = garea / grw;
+            const int chunks = (grw + kWave - 1) / kWave;
+            uint32_t* const chunk_rows = s_chunk_rows[wave];
+            for (int c = 0; c < chunks; c++) {       // union of the column spans of 64 columns: first | last << 15
+                const int x = c * kWave + lane;
+                const uint32_t col = x < grw ? spans[x] : 1u;
+                uint32_t lo = col & 0x7fffu, hi = (col >> 15) & 0x7fffu;
+                if (lo > hi) { lo = 0x7fffu; hi = 0; }
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) {
+                    lo = min(lo, (uint32_t)__shfl_xor((int)lo, o));
+                    hi = max(hi, (uint32_t)__shfl_xor((int)hi, o));
+                }
+                if (lane == 0) chunk_rows[c] = lo | (hi << 15);
+            }
+            __builtin_amdgcn_wave_barrier();
+            const int rows = (grh + kWavesPerBlock - 1) / kWavesPerBlock;
+            const int y_lo = min(grh, wave * rows), y_hi = min(grh, y_lo + rows);
+            for (int ty = y_lo; ty < y_hi; ty++) {
+                const uint32_t row = spans[grw + ty];
+                const uint32_t rlo = row & 0x7fffu, rhi = (row >> 15) & 0x7fffu;
+                for (int c = 0; c < chunks; c++) {
+                    const uint32_t cr = chunk_rows[c];
+                    const bool columns_reach = (uint32_t)ty >= (cr & 0x7fffu) && (uint32_t)ty <= ((cr >> 15) & 0x7fffu);
+                    const bool row_reaches = rlo <= rhi && rlo <= (uint32_t)(c * kWave + kWave - 1) && rhi >= (uint32_t)(c * kWave);
+                    if (!columns_reach && !row_reaches && (row >> 30) == 0) continue;
+                    const int tx = c * kWave + lane;
+                    bool ok = false;
+                    if (tx < grw) {
+                        const uint32_t col = spans[tx];
+                        const bool by_column = (uint32_t)ty >= (col & 0x7fffu) && (uint32_t)ty <= ((col >> 15) & 0x7fffu);
+                        const bool by_row = (uint32_t)tx >= rlo && (uint32_t)tx <= rhi;
+                        ok = by_column || by_row || ((col & row) >> 30) != 0;
+                    }
+                    visit(tx, ty, ok);
+                }
+            }
+        } else {
+            const int part = ((garea + kWavesPerBlock - 1) / kWavesPerBlock + kWave - 1) / kWave * kWave;
+            const int j_lo = min(garea, wave * part), j_hi = min(garea, j_lo + part);
+            for (int base = j_lo; base < j_hi; base += kWave) {
+                const int j = base + lane;
+                bool ok = false;
+                int tx = 0, ty = 0;
+                if (j < j_hi) {
+                    div_mod(j, grw, ty, tx);
+                    ok = tile_hit(gminx + tx, gminy + ty, cam.bx, cam.by, s_huge_f[e][0], s_huge_f[e][1],
+                                  s_huge_f[e][2], s_huge_f[e][3], s_huge_f[e][4], s_huge_f[e][5]);
+                }
+                visit(tx, ty, ok);
+            }
         }
-        return tile_hit(s_huge_i[e][0] + tx, s_huge_i[e][1] + ty, cam.bx, cam.by, s_huge_f[e][0], s_huge_f[e][1],
-                        s_huge_f[e][2], s_huge_f[e][3], s_huge_f[e][4], s_huge_f[e][5]);
     };
     for (int e = 0; e < n_huge; e++) {
         const bool from_spans = s_huge_spans[e] != 0;
         if (from_spans) fill_spans(e);
-        const int grw = s_huge_i[e][2], garea = s_huge_i[e][3];
-        const int part = ((garea + kWavesPerBlock - 1) / kWavesPerBlock + kWave - 1) / kWave * kWave;
-        const int j_lo = min(garea, wave * part), j_hi = min(garea, j_lo + part);
         uint32_t total = 0;
-        for (int base = j_lo; base < j_hi; base += kWave) {
-            const int j = base + lane;
-            bool ok = false;
-            if (j < j_hi) {
-                int tx, ty;
-                div_mod(j, grw, ty, tx);
-                ok = listed_tile_hit(e, from_spans, tx, ty, grw);
-            }
-            total += (uint32_t)__popcll(ballot(ok));
-        }
+        walk_listed(e, from_spans, [&](int, int, bool ok) { total += (uint32_t)__popcll(ballot(ok)); });
         if (lane == 0) s_huge_cnt[e][wave] = total;
     }
     if (n_huge > 0) {
@@ -718,21 +758,12 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         for (int e = 0; e < n_huge; e++) {
             const bool from_spans = s_huge_spans[e] != 0;
             if (from_spans) fill_spans(e);
-            const int gminx = s_huge_i[e][0], gminy = s_huge_i[e][1], grw = s_huge_i[e][2], garea = s_huge_i[e][3];
+            const int gminx = s_huge_i[e][0], gminy = s_huge_i[e][1];
             const uint32_t gdepth = s_huge_u[e][0], gidx = s_huge_u[e][1];
             uint64_t slot = s_huge_u[e][2];
             for (int w = 0; w < wave; w++) slot += s_huge_cnt[e][w];
             if (s_huge_cnt[e][wave] == 0) continue;
-            const int part = ((garea + kWavesPerBlock - 1) / kWavesPerBlock + kWave - 1) / kWave * kWave;
-            const int j_lo = min(garea, wave * part), j_hi = min(garea, j_lo + part);
-            for (int base = j_lo; base < j_hi; base += kWave) {
-                const int j = base + lane;
-                bool ok = false;
-                int tx = 0, ty = 0;
-                if (j < j_hi) {
-                    div_mod(j, grw, ty, tx);
-                    ok = listed_tile_hit(e, from_spans, tx, ty, grw);
-                }
+            walk_listed(e, from_spans, [&](int tx, int ty, bool ok) {
                 const uint64_t hits = ballot(ok);
                 if (ok) {
                     const uint64_t dst = slot + (uint64_t)popc_below(hits);
@@ -742,7 +773,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
                     }
                 }
                 slot += (uint64_t)__popcll(hits);
-            }
+            });
         }
     }
     {
