@@ -31,6 +31,7 @@ constexpr int kStashCap = 1024;         // flat candidates (and so stashed hits)
 constexpr int kHugeMin = 1024;          // rectangles with more tiles than this are tested by the whole workgroup
 constexpr int kHugeCap = 16;            // such rectangles per workgroup; further ones stay with their wave
 constexpr int kSpanWords = kWavesPerBlock * kStashCap / 4;   // column + row spans of one listed rectangle
+static_assert(kSpanWords / kWave <= kWave, "one lane per group of 64 columns");
 constexpr unsigned kSpinLimit = 1u << 22;   // polls before a chained-scan wait gives up
 
 struct Camera {
@@ -414,7 +415,6 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     __shared__ int s_huge_i[kHugeCap][4];
     __shared__ uint32_t s_huge_u[kHugeCap][3];                  // depth bits, Gaussian index, first slot
     __shared__ uint32_t s_huge_cnt[kHugeCap][kWavesPerBlock];
-    __shared__ uint32_t s_chunk_rows[kWavesPerBlock][kSpanWords / kWave];   // rows covered by the column spans of 64 columns
     __shared__ int s_huge_spans[kHugeCap];                      // 1: the tiles that pass are found from column and row spans
     __shared__ int s_nhuge;
 
@@ -635,8 +635,9 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         if (from_spans) {
             const int grh = garea / grw;
             const int chunks = (grw + kWave - 1) / kWave;
-            uint32_t* const chunk_rows = s_chunk_rows[wave];
-            for (int c = 0; c < chunks; c++) {       // union of the column spans of 64 columns: first | last << 15
+            // lane c keeps the union of the column spans of columns 64c .. 64c + 63 (first row, last row)
+            uint32_t chunk_lo = 0x7fffu, chunk_hi = 0;
+            for (int c = 0; c < chunks; c++) {
                 const int x = c * kWave + lane;
                 const uint32_t col = x < grw ? spans[x] : 1u;
                 uint32_t lo = col & 0x7fffu, hi = (col >> 15) & 0x7fffu;
@@ -646,19 +647,19 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
                     lo = min(lo, (uint32_t)__shfl_xor((int)lo, o));
                     hi = max(hi, (uint32_t)__shfl_xor((int)hi, o));
                 }
-                if (lane == 0) chunk_rows[c] = lo | (hi << 15);
+                if (lane == c) { chunk_lo = lo; chunk_hi = hi; }
             }
-            __builtin_amdgcn_wave_barrier();
             const int rows = (grh + kWavesPerBlock - 1) / kWavesPerBlock;
             const int y_lo = min(grh, wave * rows), y_hi = min(grh, y_lo + rows);
             for (int ty = y_lo; ty < y_hi; ty++) {
                 const uint32_t row = spans[grw + ty];
                 const uint32_t rlo = row & 0x7fffu, rhi = (row >> 15) & 0x7fffu;
-                for (int c = 0; c < chunks; c++) {
-                    const uint32_t cr = chunk_rows[c];
-                    const bool columns_reach = (uint32_t)ty >= (cr & 0x7fffu) && (uint32_t)ty <= ((cr >> 15) & 0x7fffu);
-                    const bool row_reaches = rlo <= rhi && rlo <= (uint32_t)(c * kWave + kWave - 1) && rhi >= (uint32_t)(c * kWave);
-                    if (!columns_reach && !row_reaches && (row >> 30) == 0) continue;
+                // one lane per chunk decides whether the step is needed; the wave walks the needed ones
+                const bool columns_reach = (uint32_t)ty >= chunk_lo && (uint32_t)ty <= chunk_hi;
+                const bool row_reaches = rlo <= rhi && rlo <= (uint32_t)(lane * kWave + kWave - 1) && rhi >= (uint32_t)(lane * kWave);
+                uint64_t needed = ballot(lane < chunks && (columns_reach || row_reaches || (row >> 30) != 0));
+                for (; needed; needed &= needed - 1) {
+                    const int c = __ffsll((long long)needed) - 1;
                     const int tx = c * kWave + lane;
                     bool ok = false;
                     if (tx < grw) {
