@@ -28,6 +28,54 @@ __global__ __launch_bounds__(256) void fill_i32_kernel(int* p, size_t n, int v)
 // kRangesPerThread pairs, 256 apart so that the loads of a workgroup stay contiguous.
 constexpr int kRangesPerThread = 8;
 
+// Tiles of a small frame ranked by the length of their lists, longest first (in steps of 16;
+// the order inside a step is whatever the atomics make it).  One workgroup.
+// (Ranking in the last workgroup of tile_ranges_kernel instead costs more than this launch: every
+// workgroup then has to push its ranges out of its XCD's L2 before it counts itself done.)
+constexpr int kOrderCap = 8192;            // tiles
+constexpr int kOrderBins = 128;            // everything from 2032 entries up shares the first bin
+__device__ uint32_t g_tile_order[kOrderCap];
+
+__global__ __launch_bounds__(1024) void tile_order_kernel(const int2* __restrict__ ranges, int num_tiles)
+{
+    constexpr int kPerThread = kOrderCap / 1024;
+    __shared__ uint32_t s_count[kOrderBins];
+    const int tid = threadIdx.x;
+    if (tid < kOrderBins) s_count[tid] = 0;
+    __syncthreads();
+    uint32_t bin[kPerThread], slot[kPerThread];
+#pragma unroll
+    for (int k = 0; k < kPerThread; k++) {
+        const int t = tid + k * 1024;
+        bin[k] = 0; slot[k] = 0;
+        if (t < num_tiles) {
+            const int2 r = ranges[t];
+            bin[k] = (uint32_t)(kOrderBins - 1 - max(0, min((r.y - r.x) >> 4, kOrderBins - 1)));
+            slot[k] = atomicAdd(&s_count[bin[k]], 1u);
+        }
+    }
+    __syncthreads();
+    if (tid < kWave) {
+        // exclusive prefix over the bins, two per lane
+        const uint32_t a = s_count[2 * tid], b = s_count[2 * tid + 1];
+        uint32_t incl = a + b;
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+            const uint32_t up = (uint32_t)__shfl_up((int)incl, o);
+            if (tid >= o) incl += up;
+        }
+        const uint32_t excl = incl - (a + b);
+        s_count[2 * tid] = excl;
+        s_count[2 * tid + 1] = excl + a;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kPerThread; k++) {
+        const int t = tid + k * 1024;
+        if (t < num_tiles) g_tile_order[s_count[bin[k]] + slot[k]] = (uint32_t)t;
+    }
+}
+
 __global__ __launch_bounds__(256) void tile_ranges_kernel(int L, const uint64_t* __restrict__ keys,
                                                           int2* __restrict__ ranges, uint32_t num_tiles)
 {
@@ -119,80 +167,75 @@ __device__ __forceinline__ void shade_quad(Quad& q, const float xy[2][2], const 
         }
 }
 
+// Lane-constant part of the walk: where this lane reads the staged records, what it stages.
 template <int SX, int SY>
-__device__ __forceinline__ void blend_tile(
-    const int2* __restrict__ ranges,
-    const uint32_t* __restrict__ point_list,
-    int width, int height, int tiles_x, int tiles_y,
+struct LaneRole {
+    static constexpr int kFx = 16 * SX, kGy = 16 * SY;
+    static constexpr int kRec = kFx + kGy + 4;  // floats per staged Gaussian: F table, G table, (cy, r, g, b)
+    uint32_t off_f, off_g, off_u;               // byte offsets into a staged record
+    int stage_slot;                             // Gaussian lane%32 of the batch
+    bool stage_g;                               // lanes 0-31 tabulate F, 32-63 G
+    float xy[SX * SY][2][2];                    // X*Y of the quad's pixels, offsets from the tile centre
+
+    __device__ __forceinline__ void init(int lane)
+    {
+        // lane -> 2x2 quad of every 16x16 sub-tile
+        const int qx = (lane & 7) * 2, qy = (lane >> 3) * 2;
+#pragma unroll
+        for (int s = 0; s < SX * SY; s++) {
+            const int lx = (s % SX) * 16 + qx, ly = (s / SX) * 16 + qy;
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int i = 0; i < 2; i++) xy[s][j][i] = (float)((lx + i - kFx / 2) * (ly + j - kGy / 2));
+        }
+        // The offsets are held in vector registers (the empty asm hides what the compiler could
+        // know about them) so that every LDS read of the unrolled batch is "register +
+        // immediate": no address arithmetic in the loop.
+        off_f = 4u * (uint32_t)qx; off_g = 4u * (uint32_t)(kFx + qy); off_u = 4u * (uint32_t)(kFx + kGy);
+        asm volatile("" : "+v"(off_f), "+v"(off_g), "+v"(off_u));
+        stage_slot = lane & (kBatch - 1);
+        stage_g = lane >= kBatch;
+    }
+};
+
+__device__ __forceinline__ void clear_quad(Quad& q)
+{
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            q.T[j][i] = 1.0f;
+            q.r[j][i] = 0.0f; q.g[j][i] = 0.0f; q.b[j][i] = 0.0f;
+        }
+}
+
+// One wave blends entries [begin, begin + n) of the sorted list into the quads of the tile whose
+// centre is given, front to back; begin must be an even distance from the start of the tile's
+// list, so that the pairs are the reference's pairs.  Returns true when the walk ended at the
+// tile-wide stop.  s_rec is this wave's staging area of kBatch records.
+template <int SX, int SY>
+__device__ __forceinline__ bool walk_list(
+    const LaneRole<SX, SY>& role, float* s_rec,
+    const uint32_t* __restrict__ point_list, int begin, int n,
+    float centre_x, float centre_y,
     const float2* __restrict__ points_xy,
     const float4* __restrict__ rgb_depth,
     const float4* __restrict__ conic_opacity,
-    float bg_r, float bg_g, float bg_b,
-    uint8_t* __restrict__ out_u8,
-    float* __restrict__ out_f32)
+    Quad (&quad)[SX * SY])
 {
     using Staged = StagedT<SX, SY>;
-    constexpr int kSub = SX * SY;              // 16x16 sub-tiles per tile = quads per lane
+    constexpr int kSub = SX * SY;
     constexpr int kFx = 16 * SX, kGy = 16 * SY;
     constexpr int kTab = kFx > kGy ? kFx : kGy;
-    constexpr int kRec = kFx + kGy + 4;        // floats per staged Gaussian: F table, G table, (cy, r, g, b)
-    __shared__ __align__(16) float s_rec[kBatch * kRec];
-
-    const int lane = threadIdx.x;
-    // Workgroup -> tile.  The hardware deals consecutive workgroups out to the 8 XCDs in turn, and
-    // every XCD has its own L2.  Neighbouring tiles share most of their Gaussians, so each XCD is
-    // given whole 8x8 blocks of tiles (its workgroups g = 8*slot + xcd walk blocks xcd, xcd+8, ...
-    // 64 tiles at a time): a Gaussian's attribute lines are then fetched into one L2 once instead
-    // of into several L2s once per tile.
-    const int group = blockIdx.x;
-    const int xcd = group & 7, slot = group >> 3;
-    const int blocks_x = (tiles_x + 7) >> 3;
-    const int block = (slot >> 6) * 8 + xcd, inner = slot & 63;
-    const int tile_x = (block % blocks_x) * 8 + (inner & 7);
-    const int tile_y = (block / blocks_x) * 8 + (inner >> 3);
-    if (tile_x >= tiles_x || tile_y >= tiles_y) return;
-    const int2 range = ranges[tile_y * tiles_x + tile_x];
-    const int n = range.y - range.x;
-    // A launch ends when its longest list ends, and a wave that shares its SIMD equally with the
-    // waves of short lists gets to its own end late: waves with long lists ask for a higher
-    // issue priority.
-    if (n > 1024) __builtin_amdgcn_s_setprio(3);
-    else if (n > 512) __builtin_amdgcn_s_setprio(2);
-    else if (n > 256) __builtin_amdgcn_s_setprio(1);
-
-    // lane -> 2x2 quad of every 16x16 sub-tile
-    const int qx = (lane & 7) * 2, qy = (lane >> 3) * 2;
-    const float centre_x = (float)(tile_x * kFx + kFx / 2), centre_y = (float)(tile_y * kGy + kGy / 2);
-    int pix_x[kSub], pix_y[kSub];
-    float xy[kSub][2][2];                      // X*Y of the quad's pixels, offsets from the tile centre
-    Quad quad[kSub];
-#pragma unroll
-    for (int s = 0; s < kSub; s++) {
-        const int lx = (s % SX) * 16 + qx, ly = (s / SX) * 16 + qy;
-        pix_x[s] = tile_x * kFx + lx;
-        pix_y[s] = tile_y * kGy + ly;
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                xy[s][j][i] = (float)((lx + i - kFx / 2) * (ly + j - kGy / 2));
-                quad[s].T[j][i] = 1.0f;
-                quad[s].r[j][i] = 0.0f; quad[s].g[j][i] = 0.0f; quad[s].b[j][i] = 0.0f;
-            }
-    }
-
-    // Byte offsets into a staged record.  They are held in vector registers (the empty asm hides
-    // what the compiler could know about them) so that every LDS read of the unrolled batch is
-    // "register + immediate": no address arithmetic in the loop.
+    constexpr int kRec = LaneRole<SX, SY>::kRec;
     const char* const rec_bytes = reinterpret_cast<const char*>(s_rec);
-    uint32_t off_f = 4u * (uint32_t)qx, off_g = 4u * (uint32_t)(kFx + qy), off_u = 4u * (uint32_t)(kFx + kGy);
-    asm volatile("" : "+v"(off_f), "+v"(off_g), "+v"(off_u));
-
-    // Staging role of this lane: Gaussian lane%32 of the batch; lanes 0-31 tabulate F, 32-63 G.
-    const int stage_slot = lane & (kBatch - 1);
-    const bool stage_g = lane >= kBatch;
+    const uint32_t off_f = role.off_f, off_g = role.off_g, off_u = role.off_u;
+    const int stage_slot = role.stage_slot;
+    const bool stage_g = role.stage_g;
     float* const stage_tab = s_rec + stage_slot * kRec + (stage_g ? kFx : 0);
     const int stage_len = stage_g ? kGy : kFx;
+    const int last = begin + n - 1;
 
     // registers hold the batch that is staged next; loads for it overlap the shading of the current one
     float2 nxy = make_float2(0.f, 0.f);
@@ -202,8 +245,8 @@ __device__ __forceinline__ void blend_tile(
     // of the list are clamped to its last entry: those loads are valid and their result unused.
     uint32_t g_ahead = 0;
     if (n > 0) {
-        const uint32_t g = point_list[min(range.x + stage_slot, range.y - 1)];
-        g_ahead = point_list[min(range.x + kBatch + stage_slot, range.y - 1)];
+        const uint32_t g = point_list[min(begin + stage_slot, last)];
+        g_ahead = point_list[min(begin + kBatch + stage_slot, last)];
         nxy = points_xy[g]; nco = conic_opacity[g]; nrgb = rgb_depth[g];
     }
 
@@ -235,7 +278,7 @@ __device__ __forceinline__ void blend_tile(
         }
         __builtin_amdgcn_wave_barrier();
         nxy = points_xy[g_ahead]; nco = conic_opacity[g_ahead]; nrgb = rgb_depth[g_ahead];
-        g_ahead = point_list[min(range.x + base + 2 * kBatch + stage_slot, range.y - 1)];
+        g_ahead = point_list[min(begin + base + 2 * kBatch + stage_slot, last)];
         // Gaussians go in pairs; the tile-wide stop is tested after each pair (render.cu:394-408)
         // The table reads of a Gaussian are issued before the Gaussian ahead of it is shaded, so
         // that a wave does not sit out the LDS latency once per Gaussian.
@@ -251,7 +294,7 @@ __device__ __forceinline__ void blend_tile(
         };
         auto shade = [&](const Staged& r) {
 #pragma unroll
-            for (int s = 0; s < kSub; s++) shade_quad(quad[s], xy[s], r.f[s % SX], r.g[s / SX], r.u);
+            for (int s = 0; s < kSub; s++) shade_quad(quad[s], role.xy[s], r.f[s % SX], r.g[s / SX], r.u);
         };
         auto all_stopped = [&]() {
             bool live = false;                      // some pixel of this lane still has T >= 1e-4
@@ -280,15 +323,23 @@ __device__ __forceinline__ void blend_tile(
         } while (0);
 #undef FGS_PAIR
     }
+    return done;
+}
 
-    // render.cu:59-73
+// render.cu:59-73
+template <int SX, int SY>
+__device__ __forceinline__ void write_tile(
+    int lane, int tile_x, int tile_y, int width, int height, const Quad (&quad)[SX * SY],
+    float bg_r, float bg_g, float bg_b, uint8_t* __restrict__ out_u8, float* __restrict__ out_f32)
+{
+    const int qx = (lane & 7) * 2, qy = (lane >> 3) * 2;
 #pragma unroll
-    for (int s = 0; s < kSub; s++)
+    for (int s = 0; s < SX * SY; s++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                const int x = pix_x[s] + i, y = pix_y[s] + j;
+                const int x = tile_x * 16 * SX + (s % SX) * 16 + qx + i, y = tile_y * 16 * SY + (s / SX) * 16 + qy + j;
                 if (x < width && y < height) {
                     const size_t pid = (size_t)width * y + x;
                     float t = quad[s].T[j][i];
@@ -306,6 +357,59 @@ __device__ __forceinline__ void blend_tile(
                     }
                 }
             }
+}
+
+// Position in the launch -> tile.  The hardware deals consecutive workgroups out to the 8 XCDs in
+// turn, and every XCD has its own L2.  Neighbouring tiles share most of their Gaussians, so each
+// XCD is given whole 8x8 blocks of tiles (its positions g = 8*slot + xcd walk blocks xcd, xcd+8,
+// ... 64 tiles at a time): a Gaussian's attribute lines are then fetched into one L2 once instead
+// of into several L2s once per tile.  False for the padding positions.
+__device__ __forceinline__ bool tile_of_position(int group, int tiles_x, int tiles_y, int* tile_x, int* tile_y)
+{
+    const int xcd = group & 7, slot = group >> 3;
+    const int blocks_x = (tiles_x + 7) >> 3;
+    const int block = (slot >> 6) * 8 + xcd, inner = slot & 63;
+    *tile_x = (block % blocks_x) * 8 + (inner & 7);
+    *tile_y = (block / blocks_x) * 8 + (inner >> 3);
+    return *tile_x < tiles_x && *tile_y < tiles_y;
+}
+
+template <int SX, int SY>
+__device__ __forceinline__ void blend_tile(
+    const int2* __restrict__ ranges,
+    const uint32_t* __restrict__ point_list,
+    int width, int height, int tiles_x, int tiles_y,
+    const float2* __restrict__ points_xy,
+    const float4* __restrict__ rgb_depth,
+    const float4* __restrict__ conic_opacity,
+    float bg_r, float bg_g, float bg_b,
+    uint8_t* __restrict__ out_u8,
+    float* __restrict__ out_f32)
+{
+    constexpr int kSub = SX * SY;              // 16x16 sub-tiles per tile = quads per lane
+    constexpr int kFx = 16 * SX, kGy = 16 * SY;
+    __shared__ __align__(16) float s_rec[kBatch * LaneRole<SX, SY>::kRec];
+
+    const int lane = threadIdx.x;
+    int tile_x, tile_y;
+    if (!tile_of_position((int)blockIdx.x, tiles_x, tiles_y, &tile_x, &tile_y)) return;
+    const int2 range = ranges[tile_y * tiles_x + tile_x];
+    const int n = range.y - range.x;
+    // A launch ends when its longest list ends, and a wave that shares its SIMD equally with the
+    // waves of short lists gets to its own end late: waves with long lists ask for a higher
+    // issue priority.
+    if (n > 1024) __builtin_amdgcn_s_setprio(3);
+    else if (n > 512) __builtin_amdgcn_s_setprio(2);
+    else if (n > 256) __builtin_amdgcn_s_setprio(1);
+
+    LaneRole<SX, SY> role;
+    role.init(lane);
+    Quad quad[kSub];
+#pragma unroll
+    for (int s = 0; s < kSub; s++) clear_quad(quad[s]);
+    const float centre_x = (float)(tile_x * kFx + kFx / 2), centre_y = (float)(tile_y * kGy + kGy / 2);
+    walk_list<SX, SY>(role, s_rec, point_list, range.x, n, centre_x, centre_y, points_xy, rgb_depth, conic_opacity, quad);
+    write_tile<SX, SY>(lane, tile_x, tile_y, width, height, quad, bg_r, bg_g, bg_b, out_u8, out_f32);
 }
 
 #define FGS_BLEND_PARAMS                                                                         \
@@ -333,6 +437,116 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4, 4))) v
 {
     blend_tile<SX, SY>(FGS_BLEND_ARGS);
 }
+
+// For a frame that is resident at once, one wave per tile means that the launch lasts as long as
+// the longest list.  Here a workgroup of four waves takes four tiles that lie far apart (a long
+// list then usually has three short neighbours): every wave blends the first kOwnShare entries of
+// its own tile, and what is left of a tile after that is cut into four runs of pairs, one per
+// wave.  A run is blended from T = 1, C = 0 and the owner folds the runs in front-to-back order,
+// C += T C_run, T *= T_run, which is the same sum in another order of additions.  A run stops
+// when its own T is below the threshold everywhere, so a tile can be walked a little further than
+// the reference walks it: what that adds is below 1e-4 of a colour.
+constexpr int kOwnShare = 256;
+constexpr int kMinRest = 512;               // a shorter rest is not worth two barriers: the owner walks it
+constexpr int kSharedWaves = 4;
+
+__global__ __launch_bounds__(kSharedWaves * kWave) void blend_kernel_shared(FGS_BLEND_PARAMS)
+{
+    using Role = LaneRole<1, 1>;
+    __shared__ __align__(16) float s_rec[kSharedWaves][kBatch * Role::kRec];
+    __shared__ int s_rest[kSharedWaves], s_from[kSharedWaves], s_tile_x[kSharedWaves], s_tile_y[kSharedWaves];
+    static_assert(kBatch * Role::kRec >= 4 * 4 * kWave, "a run's result (4 pixels x 4 floats per lane) is handed over in the staging area");
+
+    const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    // Wave w takes rank g of quarter w of the tiles ranked by list length: the workgroups with
+    // the longest lists come first in the launch, and a long list has three shorter ones beside it.
+    const int rank = wave * (int)gridDim.x + (int)blockIdx.x;
+    const bool active = rank < tiles_x * tiles_y;
+    int tile_x = 0, tile_y = 0;
+    if (active) {
+        const int tile = (int)g_tile_order[rank];
+        tile_x = tile % tiles_x;
+        tile_y = tile / tiles_x;
+    }
+    int2 range = make_int2(0, 0);
+    if (active) range = ranges[tile_y * tiles_x + tile_x];
+    const int n = range.y - range.x;
+    if (n > 256) __builtin_amdgcn_s_setprio(1);
+
+    Role role;
+    role.init(lane);
+    if (lane == 0) {
+        s_rest[wave] = n;               // job 0 of wave w: the head of its own list, in one run
+        s_from[wave] = range.x;
+        s_tile_x[wave] = tile_x;
+        s_tile_y[wave] = tile_y;
+    }
+    // job 0: own head; job 1 + v: this wave's run of what is left of tile v.  While a wave blends
+    // runs, the result of its own head waits in its private memory, not in registers.
+    Quad part[1];
+    volatile float kept[16];
+    bool shared_out = false;
+    for (int job = 0; job <= kSharedWaves; job++) {
+        const int v = job == 0 ? wave : job - 1;
+        const int rest = __builtin_amdgcn_readfirstlane(s_rest[v]);
+        if (job != 0 && rest == 0) continue;
+        int skip = 0, count = rest > kOwnShare + kMinRest ? kOwnShare : rest;
+        if (job != 0) {
+            const int run = (((rest + kSharedWaves - 1) / kSharedWaves) + 1) & ~1;      // whole pairs
+            skip = min(wave * run, rest);
+            count = min(run, rest - skip);
+        }
+        clear_quad(part[0]);
+        const bool stopped = walk_list<1, 1>(role, s_rec[wave], point_list, __builtin_amdgcn_readfirstlane(s_from[v]) + skip, count,
+                                             (float)(__builtin_amdgcn_readfirstlane(s_tile_x[v]) * 16 + 8),
+                                             (float)(__builtin_amdgcn_readfirstlane(s_tile_y[v]) * 16 + 8),
+                                             points_xy, rgb_depth, conic_opacity, part);
+        if (job == 0) {
+            if (lane == 0) {
+                s_rest[wave] = (!stopped && n > kOwnShare + kMinRest) ? n - kOwnShare : 0;
+                s_from[wave] = range.x + kOwnShare;
+            }
+            __syncthreads();
+            shared_out = (s_rest[0] | s_rest[1] | s_rest[2] | s_rest[3]) != 0;
+            if (!shared_out) break;
+            __builtin_amdgcn_s_setprio(3);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                kept[4 * k + 0] = part[0].r[k >> 1][k & 1]; kept[4 * k + 1] = part[0].g[k >> 1][k & 1];
+                kept[4 * k + 2] = part[0].b[k >> 1][k & 1]; kept[4 * k + 3] = part[0].T[k >> 1][k & 1];
+            }
+            continue;
+        }
+        float4* const mine = reinterpret_cast<float4*>(s_rec[wave]);
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            mine[k * kWave + lane] = make_float4(part[0].r[k >> 1][k & 1], part[0].g[k >> 1][k & 1],
+                                                 part[0].b[k >> 1][k & 1], part[0].T[k >> 1][k & 1]);
+        __syncthreads();
+        if (wave == v) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float r = kept[4 * k + 0], g = kept[4 * k + 1], b = kept[4 * k + 2], t = kept[4 * k + 3];
+#pragma unroll
+                for (int w = 0; w < kSharedWaves; w++) {
+                    const float4 p = reinterpret_cast<const float4*>(s_rec[w])[k * kWave + lane];
+                    r += t * p.x; g += t * p.y; b += t * p.z;
+                    t *= p.w;
+                }
+                kept[4 * k + 0] = r; kept[4 * k + 1] = g; kept[4 * k + 2] = b; kept[4 * k + 3] = t;
+            }
+        }
+        __syncthreads();
+    }
+    if (shared_out) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            part[0].r[k >> 1][k & 1] = kept[4 * k + 0]; part[0].g[k >> 1][k & 1] = kept[4 * k + 1];
+            part[0].b[k >> 1][k & 1] = kept[4 * k + 2]; part[0].T[k >> 1][k & 1] = kept[4 * k + 3];
+        }
+    }
+    if (active) write_tile<1, 1>(lane, tile_x, tile_y, width, height, part, bg_r, bg_g, bg_b, out_u8, out_f32);
+}
 #undef FGS_BLEND_PARAMS
 #undef FGS_BLEND_ARGS
 
@@ -344,6 +558,25 @@ int check_tile(int block_x, int block_y, int* sx, int* sy, const char* who)
         return FGS_OK;
     }
     return fail(FGS_E_INVALID, "%s: tile %dx%d unsupported (16x16, 32x16, 32x32)", who, block_x, block_y);
+}
+
+// How a frame is blended.  More tiles than the chip holds at 8 waves per SIMD: the variant with
+// fewer resident waves.  A frame of 16x16 tiles that is resident at once: workgroups of four tiles
+// that share out their long lists, which needs the tiles ranked by list length.
+struct BlendShape {
+    int cus;
+    bool few_waves, shared;
+};
+
+int blend_shape(int block_x, int block_y, int tiles_x, int tiles_y, BlendShape* shape)
+{
+    int dev = 0;
+    FGS_HIP_TRY(hipGetDevice(&dev));
+    FGS_HIP_TRY(hipDeviceGetAttribute(&shape->cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const long long num_tiles = (long long)tiles_x * tiles_y;
+    shape->few_waves = num_tiles > 32LL * shape->cus;
+    shape->shared = !shape->few_waves && block_x == 16 && block_y == 16 && num_tiles <= kOrderCap && shape->cus > 0;
+    return FGS_OK;
 }
 
 // render.cu:556-563: zero the ranges, then mark where each tile starts and ends
@@ -393,11 +626,10 @@ int blend_impl(int block_x, int block_y, int width, int height,
     const long long groups = (blocks + 7) / 8 * 8 * 64;
     if (groups > 0x7fffffffLL) return fail(FGS_E_INVALID, "%s: image too large", who);
     const dim3 grid((unsigned)groups);
-    // more tiles than the chip holds at 8 waves per SIMD: run the variant with fewer resident waves
-    int dev = 0, cus = 0;
-    FGS_HIP_TRY(hipGetDevice(&dev));
-    FGS_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    const bool few_waves = (long long)tiles_x * tiles_y > 32LL * cus;
+    BlendShape shape;
+    rc = blend_shape(block_x, block_y, tiles_x, tiles_y, &shape);
+    if (rc != FGS_OK) return rc;
+    const bool few_waves = shape.few_waves;
 #define FGS_LAUNCH_BLEND(SX, SY)                                                                        \
     do {                                                                                                \
         auto kernel = few_waves ? blend_kernel_few_waves<SX, SY> : blend_kernel<SX, SY>;                \
@@ -406,7 +638,14 @@ int blend_impl(int block_x, int block_y, int width, int height,
                            (const float2*)points_xy, (const float4*)rgb_depth, (const float4*)conic_opacity, \
                            bg[0], bg[1], bg[2], out_u8, out_f32);                                       \
     } while (0)
-    if (sx == 1 && sy == 1) FGS_LAUNCH_BLEND(1, 1);
+    if (shape.shared) {
+        const int num_tiles = tiles_x * tiles_y;
+        hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, st, (const int2*)ranges, num_tiles);
+        hipLaunchKernelGGL(blend_kernel_shared, dim3((unsigned)((num_tiles + kSharedWaves - 1) / kSharedWaves)), dim3(kSharedWaves * kWave), 0, st,
+                           (const int2*)ranges, values_sorted, width, height, tiles_x, tiles_y,
+                           (const float2*)points_xy, (const float4*)rgb_depth, (const float4*)conic_opacity,
+                           bg[0], bg[1], bg[2], out_u8, out_f32);
+    } else if (sx == 1 && sy == 1) FGS_LAUNCH_BLEND(1, 1);
     else if (sx == 2 && sy == 1) FGS_LAUNCH_BLEND(2, 1);
     else FGS_LAUNCH_BLEND(2, 2);
 #undef FGS_LAUNCH_BLEND

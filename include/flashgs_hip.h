@@ -86,6 +86,12 @@ size_t fgs_get_sort_buffer_size(int num_rendered);
  * csrc/cuda_rasterizer/render.cu:549-608): zero `ranges`, find each tile's [start,end) in the
  * sorted keys, blend front to back and write out_color u8[H,W,3].  `ranges` int32[tiles,2] is
  * scratch that holds the tile ranges afterwards.  bg_color is a host array of 3 floats.
+ * A frame of at most 8192 16x16 tiles first ranks its tiles by list length into a table the
+ * library keeps per device (4 bytes per tile), and the rest of a list of more than 768 entries
+ * is blended in four runs that each stop on their own transmittance: the colour can differ from
+ * the pair-by-pair walk of render.cu:315-408 by what lies behind T < 1e-4, i.e. by less than
+ * 1e-4 of a colour.  Because of the table, blends on one device must not overlap in time (calls
+ * on one stream, or otherwise ordered, never do).
  */
 int fgs_render_16x16(int num_rendered, int width, int height,
                      const float* points_xy, const float* rgb_depth, const float* conic_opacity,

@@ -388,6 +388,59 @@ def test_sort_full_size_properties():
     assert int(torch.bincount(vs.long(), minlength=n).max()) == 1     # a permutation
 
 
+def test_blend_long_lists_shared_between_waves(oracle):
+    """A small frame blends its long lists with four waves: the owner takes the head of the list,
+    the rest is cut into four runs that start from T = 1 and are folded front to back.  Crafted
+    lists around the lengths where that sets in, with odd and even lengths, one that saturates in
+    its head, one that saturates inside a run and faint ones that never do; blended through
+    fgs_blend on ranges made here, against the oracle's blend of the same lists."""
+    import gpu_pipeline as gp
+    from flashgs_amd import cabi
+    import torch
+    W, H = 320, 232                      # 20 x 15 tiles, the last row half a tile
+    gx, gy = 20, 15
+    rng = np.random.default_rng(11)
+    # (tile, list length, opacity): faint lists never reach the stop
+    lists = [(0, 767, 0.002), (21, 768, 0.002), (22, 769, 0.002), (45, 770, 0.002), (66, 1501, 0.002),
+             (107, 3000, 0.0015), (150, 5003, 0.001), (171, 2000, 0.9), (212, 2000, 0.02), (253, 1024, 0.004),
+             (299, 900, 0.003), (280, 2048, 0.002)]
+    lists += [(t, int(rng.integers(0, 300)), 0.05) for t in range(300) if t not in {l[0] for l in lists}]
+    xy, co, rgbd, vals, ranges = [], [], [], [], np.zeros((gx * gy, 2), np.int32)
+    at = 0
+    for t, n, op in sorted(lists):
+        tx, ty = t % gx, t // gx
+        c = np.stack([tx * 16 + rng.uniform(-4, 20, n), ty * 16 + rng.uniform(-4, 20, n)], 1)
+        sig = rng.uniform(3.0, 12.0, (n, 2))
+        rho = rng.uniform(-0.6, 0.6, n)
+        det = (sig[:, 0] * sig[:, 1]) ** 2 * (1 - rho ** 2)
+        cx, cz = sig[:, 1] ** 2 / det, sig[:, 0] ** 2 / det
+        cy = -rho * sig[:, 0] * sig[:, 1] / det
+        log2e = 1.4426950408889634
+        xy.append(c)
+        co.append(np.stack([-0.5 * log2e * cx, -log2e * cy, -0.5 * log2e * cz, np.log2(np.full(n, op))], 1))
+        rgbd.append(np.concatenate([rng.uniform(0, 1.5, (n, 3)), rng.uniform(1, 50, (n, 1))], 1))
+        ranges[t] = (at, at + n)
+        at += n
+    xy = np.concatenate(xy).astype(np.float32)
+    co = np.concatenate(co).astype(np.float32)
+    rgbd = np.concatenate(rgbd).astype(np.float32)
+    vals = rng.permutation(at).astype(np.uint32)          # list position -> Gaussian index
+    inv = np.empty(at, np.int64); inv[vals] = np.arange(at)
+    xy_g, co_g, rgbd_g = xy[inv], co[inv], rgbd[inv]      # attributes by Gaussian index
+    bg = np.array([0.2, 0.4, 0.6], np.float32)
+    _, ref, walked = oracle.render(W, H, 16, 16, xy_g, rgbd_g, co_g, vals, ranges, bg, want_u8=False)
+    assert walked < at                                     # the opaque lists did stop early
+    out = torch.full((H, W, 3), -1.0, device=gp.DEV, dtype=torch.float32)
+    d = [gp.dev(a) for a in (xy_g, rgbd_g, co_g)]
+    dv, dr = gp.dev(vals.view(np.int32)), gp.dev(ranges)
+    for _ in range(2):                                     # the second call reuses the tile ranking buffer
+        cabi.blend(16, 16, W, H, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), dv.data_ptr(), dr.data_ptr(),
+                   bg, 0, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        err = np.abs(out.cpu().numpy() - ref)
+        assert err.max() <= 5e-4, "max abs image error %g" % err.max()
+
+
 def test_ranges_kernel_against_searchsorted():
     import gpu_pipeline as gp
     import torch
