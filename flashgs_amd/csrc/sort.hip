@@ -317,13 +317,29 @@ __global__ __launch_bounds__(256) void segment_starts_kernel(const uint64_t* __r
             before[k] = i == 0 ? 0u : ((uint32_t)(keys[i - 1] >> 32) & tile_mask) + 1u;
         }
     }
+    // A run of up to kOwnFill entries is written by the thread that found it; a longer one (a band
+    // of empty tiles, and the ids behind the last pair) by the whole wave, 64 entries per step.
+    constexpr uint32_t kOwnFill = 4;
+    const int lane = threadIdx.x & (kWave - 1);
+    auto fill_by_wave = [&](bool mine, uint32_t lo, uint32_t hi, int value) {
+        for (uint64_t todo = ballot(mine); todo; todo &= todo - 1) {
+            const int src = __ffsll((long long)todo) - 1;
+            const uint32_t from = (uint32_t)__shfl((int)lo, src), to = (uint32_t)__shfl((int)hi, src);
+            const int what = __shfl(value, src);
+            for (uint32_t v = from + (uint32_t)lane; v <= to; v += kWave) seg_start[v] = what;
+        }
+    };
 #pragma unroll
     for (int k = 0; k < kStartsPerThread; k++) {
         const long long i = base + k * 256;
-        if (i >= n) break;
-        for (uint32_t v = before[k]; v <= cur[k]; v++) seg_start[v] = (int)i;     // empty loop when the field repeats
-        if (i == n - 1)
-            for (uint32_t v = cur[k] + 1; v <= ids; v++) seg_start[v] = n;
+        const bool valid = i < n;
+        // ids before[k]..cur[k] start at pair i: nothing to do when the field repeats
+        const bool some = valid && before[k] <= cur[k];
+        const bool longer = some && cur[k] - before[k] >= kOwnFill;
+        if (some && !longer)
+            for (uint32_t v = before[k]; v <= cur[k]; v++) seg_start[v] = (int)i;
+        fill_by_wave(longer, before[k], cur[k], (int)i);
+        fill_by_wave(valid && i == n - 1 && cur[k] < ids, cur[k] + 1, ids, n);
     }
 }
 
