@@ -24,9 +24,6 @@ __global__ __launch_bounds__(256) void fill_i32_kernel(int* p, size_t n, int v)
     for (; i < n; i += stride) p[i] = v;
 }
 
-// render.cu:9-31, with the tile index checked against the number of tiles.  A thread looks at
-// kRangesPerThread pairs, 256 apart so that the loads of a workgroup stay contiguous.
-constexpr int kRangesPerThread = 8;
 
 // Tiles of a small frame ranked by the length of their lists, longest first (in steps of 16;
 // the order inside a step is whatever the atomics make it).  One workgroup.
@@ -76,32 +73,54 @@ __global__ __launch_bounds__(1024) void tile_order_kernel(const int2* __restrict
     }
 }
 
+// render.cu:9-31, with the tile index checked against the number of tiles.  A thread looks at
+// kRangesPerThread pairs, 256 apart so that the loads of a workgroup stay contiguous.
+// Also writes (0, 0) for the tiles without pairs (the reference clears the whole table first,
+// render.cu:557): the pair that opens tile c clears the tiles between its predecessor's tile and
+// c, the first pair those before it and the last pair those behind it.  A run of up to 4 tiles is
+// cleared by the thread that found it, a longer one by its whole wave.
+constexpr int kRangesPerThread = 8;
+
 __global__ __launch_bounds__(256) void tile_ranges_kernel(int L, const uint64_t* __restrict__ keys,
                                                           int2* __restrict__ ranges, uint32_t num_tiles)
 {
     const long long base = (long long)blockIdx.x * (256 * kRangesPerThread) + threadIdx.x;
+    const int lane = threadIdx.x & (kWave - 1);
     uint32_t cur[kRangesPerThread], prev[kRangesPerThread];
 #pragma unroll
     for (int k = 0; k < kRangesPerThread; k++) {
         const long long idx = base + k * 256;
         cur[k] = 0; prev[k] = 0;
         if (idx < L) {
-            cur[k] = (uint32_t)(keys[idx] >> 32);
-            if (idx > 0) prev[k] = (uint32_t)(keys[idx - 1] >> 32);
+            cur[k] = min((uint32_t)(keys[idx] >> 32), num_tiles);           // num_tiles: outside the image
+            if (idx > 0) prev[k] = min((uint32_t)(keys[idx - 1] >> 32), num_tiles);
         }
     }
+    auto clear_by_wave = [&](bool mine, uint32_t lo, uint32_t hi) {         // tiles [lo, hi)
+        for (uint64_t todo = ballot(mine); todo; todo &= todo - 1) {
+            const int src = __ffsll((long long)todo) - 1;
+            const uint32_t from = (uint32_t)__shfl((int)lo, src), to = (uint32_t)__shfl((int)hi, src);
+            for (uint32_t t = from + (uint32_t)lane; t < to; t += kWave) ranges[t] = make_int2(0, 0);
+        }
+    };
 #pragma unroll
     for (int k = 0; k < kRangesPerThread; k++) {
         const long long idx = base + k * 256;
-        if (idx >= L) break;
-        if (cur[k] >= num_tiles) continue;
-        if (idx == 0) {
-            ranges[cur[k]].x = 0;
-        } else if (cur[k] != prev[k]) {
-            if (prev[k] < num_tiles) ranges[prev[k]].y = (int)idx;
-            ranges[cur[k]].x = (int)idx;
+        const bool valid = idx < L;
+        const bool opens = valid && (idx == 0 || cur[k] != prev[k]);
+        if (opens) {
+            if (idx > 0 && prev[k] < num_tiles) ranges[prev[k]].y = (int)idx;
+            if (cur[k] < num_tiles) ranges[cur[k]].x = (int)idx;
         }
-        if (idx == L - 1) ranges[cur[k]].y = L;
+        if (valid && idx == L - 1 && cur[k] < num_tiles) ranges[cur[k]].y = L;
+        // empty tiles in front of this pair's tile
+        const uint32_t lo = idx == 0 ? 0u : min(prev[k] + 1u, num_tiles);
+        const bool gap = opens && lo < cur[k];
+        const bool wide = gap && cur[k] - lo > 4u;
+        if (gap && !wide)
+            for (uint32_t t = lo; t < cur[k]; t++) ranges[t] = make_int2(0, 0);
+        clear_by_wave(wide, lo, cur[k]);
+        clear_by_wave(valid && idx == L - 1 && cur[k] + 1u < num_tiles, cur[k] + 1u, num_tiles);
     }
 }
 
@@ -595,8 +614,9 @@ int ranges_impl(int block_x, int block_y, int num_rendered, int width, int heigh
     const size_t words = num_tiles * 2;
     size_t fill_blocks = (words + 1023) / 1024;
     if (fill_blocks > 1024) fill_blocks = 1024;
-    hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)fill_blocks), dim3(256), 0, st, ranges, words, 0);
-    if (num_rendered > 0)
+    if (num_rendered == 0)
+        hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)fill_blocks), dim3(256), 0, st, ranges, words, 0);
+    else
         hipLaunchKernelGGL(tile_ranges_kernel,
                            dim3((unsigned)(((size_t)num_rendered + 256 * kRangesPerThread - 1) / (256 * kRangesPerThread))),
                            dim3(256), 0, st,

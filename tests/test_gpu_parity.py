@@ -448,9 +448,13 @@ def test_ranges_kernel_against_searchsorted():
     rng = np.random.default_rng(33)
     W, H = 1920, 1080
     tiles = 120 * 68
-    for n in (0, 1, 5, 70_001):
-        tile = np.sort(rng.integers(0, tiles, n)).astype(np.uint64)
+    for n, top, beyond in ((0, tiles, 0), (1, tiles, 0), (5, tiles, 0), (70_001, tiles, 0), (3000, tiles - 700, 0),
+                           (70_001, tiles - 3, 40)):
+        # tiles 1000..1300 and everything from `top` up stay empty; `beyond` pairs carry tile ids
+        # outside the image (they sort to the end and belong to no range)
+        tile = np.sort(rng.integers(0, top, n)).astype(np.uint64)
         tile = tile[(tile < 1000) | (tile > 1300)]
+        tile = np.concatenate([tile, np.sort(rng.integers(tiles, tiles + 9, beyond)).astype(np.uint64)])
         n = tile.size
         keys = (tile << np.uint64(32)) | rng.integers(0, 1 << 32, n).astype(np.uint64)
         dk = gp.dev(keys.view(np.int64)) if n else torch.zeros(1, device=gp.DEV, dtype=torch.int64)
