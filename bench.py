@@ -125,7 +125,7 @@ def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build renders on one GPU only; --gpus %d is not supported "
-              "(frames and tile bands are independent, see DESIGN.md for how the path would shard)" % args.gpus,
+              "(a frame shards by poses or by bands of tiles, with no exchange but the final image)" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
 

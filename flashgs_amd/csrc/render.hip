@@ -500,6 +500,7 @@ __global__ __launch_bounds__(kSharedWaves * kWave) void blend_kernel_shared(FGS_
         s_tile_x[wave] = tile_x;
         s_tile_y[wave] = tile_y;
     }
+    __builtin_amdgcn_wave_barrier();    // job 0 reads these back in the same wave; the others after the barrier below
     // job 0: own head; job 1 + v: this wave's run of what is left of tile v.  While a wave blends
     // runs, the result of its own head waits in its private memory, not in registers.
     Quad part[1];
