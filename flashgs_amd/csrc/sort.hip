@@ -110,16 +110,22 @@ __global__ __launch_bounds__(kBins) void chunk_sum_kernel(const uint32_t* __rest
     chunk_sums[(size_t)blockIdx.x * kBins + d] = s;
 }
 
-__global__ __launch_bounds__(kBins) void offsets_kernel(uint32_t* __restrict__ hist, int tiles, int chunk,
-                                                        const uint32_t* __restrict__ chunk_sums, int chunks)
+// One workgroup per chunk, up to kOffsetGroups threads per digit (blockDim.x / kBins of them): the
+// chunk sums are few and the loop over them is latency-bound, so each group of kBins threads
+// takes every groups-th batch of 16 independent loads.
+constexpr int kOffsetGroups = 4;
+
+__global__ __launch_bounds__(kBins * kOffsetGroups) void offsets_kernel(uint32_t* __restrict__ hist, int tiles, int chunk,
+                                                                        const uint32_t* __restrict__ chunk_sums, int chunks)
 {
+    __shared__ uint32_t s_total[kOffsetGroups][kBins], s_before[kOffsetGroups][kBins];
     __shared__ uint32_t s_wave[kBins / kWave];
-    const int d = threadIdx.x;
+    const int d = threadIdx.x & (kBins - 1), group = threadIdx.x / kBins;
     const int lane = d & (kWave - 1), wave = d / kWave;
     const int mine = (int)blockIdx.x;
+    const int groups = (int)blockDim.x / kBins;
     uint32_t total = 0, before = 0;
-    // batches of 16 independent loads: the chunk sums are few and the loop is latency-bound
-    for (int c0 = 0; c0 < chunks; c0 += 16) {
+    for (int c0 = group * 16; c0 < chunks; c0 += 16 * groups) {
         uint32_t v[16];
 #pragma unroll
         for (int j = 0; j < 16; j++) v[j] = c0 + j < chunks ? chunk_sums[(size_t)(c0 + j) * kBins + d] : 0u;
@@ -129,10 +135,18 @@ __global__ __launch_bounds__(kBins) void offsets_kernel(uint32_t* __restrict__ h
             total += v[j];
         }
     }
-    // exclusive scan of the digit totals over the 256 digits
-    uint32_t incl = wave_inclusive_sum(total);
-    if (lane == kWave - 1) s_wave[wave] = incl;
+    s_total[group][d] = total;
+    s_before[group][d] = before;
     __syncthreads();
+    total = 0; before = 0;
+#pragma unroll
+    for (int g = 0; g < kOffsetGroups; g++)
+        if (g < groups) { total += s_total[g][d]; before += s_before[g][d]; }
+    // exclusive scan of the digit totals over the 256 digits (every group does the same sums)
+    uint32_t incl = wave_inclusive_sum(total);
+    if (group == 0 && lane == kWave - 1) s_wave[wave] = incl;
+    __syncthreads();
+    if (group != 0) return;
     uint32_t digit_base = incl - total;
     for (int w = 0; w < wave; w++) digit_base += s_wave[w];
 
@@ -881,7 +895,7 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         const int nbits = tile_bits - 8 * p < 8 ? tile_bits - 8 * p : 8;
         hipLaunchKernelGGL(count_kernel, dim3(ws.tiles), dim3(kSortBlock), 0, st, src_k, n, shift, nbits, hist);
         hipLaunchKernelGGL(chunk_sum_kernel, dim3(ws.chunks), dim3(kBins), 0, st, hist, ws.tiles, ws.chunk, chunk_sums);
-        hipLaunchKernelGGL(offsets_kernel, dim3(ws.chunks), dim3(kBins), 0, st, hist, ws.tiles, ws.chunk, chunk_sums, ws.chunks);
+        hipLaunchKernelGGL(offsets_kernel, dim3(ws.chunks), dim3(kBins * (ws.chunks > 16 ? kOffsetGroups : 1)), 0, st, hist, ws.tiles, ws.chunk, chunk_sums, ws.chunks);
         hipLaunchKernelGGL(scatter_kernel, dim3(ws.tiles), dim3(kSortBlock), 0, st,
                            src_k, src_v, dst_k, dst_v, n, shift, nbits, hist);
         src_k = dst_k;
