@@ -30,7 +30,7 @@ FP32_PEAK_TFLOPS = 157.3         # MI355X fp32 vector, published (packed FMA)
 LANE_SLOTS_PER_S = 256 * 4 * 16 * 2.4e9   # VALU issue slots per second without packed math
 # HBM bytes per blend launch on the headline configuration, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE scaled by the readings of a 256 MiB copy (profiles/frame_cfg2_4K_hbm_traffic.txt); other workloads: not measured
-BLEND_TRAFFIC_BYTES = {"cfg2_3M_4K": 1041668880}
+BLEND_TRAFFIC_BYTES = {"cfg2_3M_4K": 1041157041}
 FLOP_PER_EVAL = 19               # render.cu:40-52: 2 sub, 6 mul + 3 add, 1 mul, 3 FMA, 1 sub
 SLOTS_PER_EVAL = 17              # 13 VALU with FMA contraction + a quarter-rate exp2 (the reference formulation)
 
