@@ -832,6 +832,7 @@ __global__ __launch_bounds__(kSortBlock) void segment_sort_general_kernel(
 }
 
 constexpr int kCapTiny = 512, kCapSmall = 1024, kCapMedium = 4096, kCapLarge = 8192;
+constexpr uint32_t kOneLaunchIds = 16384;    // up to this many tile ids one launch sorts every segment of up to kCapSmall pairs
 
 
 } // namespace
@@ -935,12 +936,23 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         // Up to 512 pairs: one wave, bitonic network in registers; one tile id per wave (neighbouring
         // tiles tend to be equally busy, so a wave that took several of them would become the tail
         // of the launch).  With a table the launch also lists the longer segments.
-        hipLaunchKernelGGL((segment_sort_wave_kernel<kCapTiny / kWave, 1>), dim3(ids), dim3(kWave),
-                           0, st, ks, vs, n, tile_mask, 1, ids, (const int*)seg_start, seg_flags,
-                           kCapSmall, kCapMedium, kCapLarge, seg_counts, seg_start ? list_small : nullptr, list_medium,
-                           list_large, cap_small, cap_medium, cap_large);
+        // A frame of few tiles has few segments of 513..1024 pairs, about one wave per SIMD, and a
+        // launch of their own lasts as long as one such sort: there the first launch takes them
+        // too, with 16 register slots (1080p: -15 us; at 4K no difference, at 8K +65 us, because
+        // the launch over 131 072 ids then runs at 3 instead of 7 waves per SIMD).
+        const bool one_wave_launch = seg_start && ids <= kOneLaunchIds;
+        if (one_wave_launch)
+            hipLaunchKernelGGL((segment_sort_wave_kernel<kCapSmall / kWave, 1>), dim3(ids), dim3(kWave),
+                               0, st, ks, vs, n, tile_mask, 1, ids, (const int*)seg_start, seg_flags,
+                               kCapSmall, kCapMedium, kCapLarge, seg_counts, list_small, list_medium,
+                               list_large, cap_small, cap_medium, cap_large);
+        else
+            hipLaunchKernelGGL((segment_sort_wave_kernel<kCapTiny / kWave, 1>), dim3(ids), dim3(kWave),
+                               0, st, ks, vs, n, tile_mask, 1, ids, (const int*)seg_start, seg_flags,
+                               kCapSmall, kCapMedium, kCapLarge, seg_counts, seg_start ? list_small : nullptr, list_medium,
+                               list_large, cap_small, cap_medium, cap_large);
         if (seg_start) {
-            if (n > kCapTiny)       // 513..1024: the same network over 16 register slots, from the lists
+            if (n > kCapTiny && !one_wave_launch)       // 513..1024: the same network over 16 register slots, from the lists
                 hipLaunchKernelGGL((segment_sort_wave_list_kernel<kCapSmall / kWave>),
                                    dim3(list_grid((unsigned)(n / (kCapTiny + 1) + 1), 8192u)),
                                    dim3(kWave), 0, st, ks, vs, (const int*)seg_start, seg_flags,
