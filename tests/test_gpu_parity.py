@@ -509,14 +509,15 @@ def test_sort_segment_size_classes(seg):
     _sort_case(tile, depth.view(np.uint32), W, H, seed=seg)
 
 
-def test_sort_every_segment_length_up_to_1100():
+@pytest.mark.parametrize("W,H", [(1920, 1080), (3840, 2160)])
+def test_sort_every_segment_length_up_to_1100(W, H):
     """One tile per length 1 ... 1100: every padding of the register sorting networks (64, 128, ... 1024
     elements) and the first lengths of the next class, with many equal depths (ties must keep input
-    order) and with depths of all magnitudes, 0 and 0xffffffff included."""
+    order) and with depths of all magnitudes, 0 and 0xffffffff included.  At 1080p one launch sorts
+    every segment of up to 1024 pairs, at 4K those above 512 come from a list in a launch of their own."""
     rng = np.random.default_rng(1100)
-    W, H = 1920, 1080
     lengths = np.arange(1, 1101)
-    tiles = rng.permutation(120 * 68)[:lengths.size].astype(np.uint32)
+    tiles = rng.permutation(((W + 15) // 16) * ((H + 15) // 16))[:lengths.size].astype(np.uint32)
     tile = np.repeat(tiles, lengths)
     depth = rng.integers(0, 1 << 32, tile.size, dtype=np.uint64).astype(np.uint32)
     depth[::5] = depth[1::5][: depth[::5].size]          # duplicates next to each other before the shuffle
