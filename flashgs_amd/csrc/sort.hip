@@ -164,6 +164,33 @@ __global__ __launch_bounds__(kBins * kOffsetGroups) void offsets_kernel(uint32_t
     }
 }
 
+// The same for a short list (at most kSmallRows histogram rows): one workgroup, one thread per
+// digit, no chunk sums in between.
+constexpr int kSmallRows = 64;
+
+__global__ __launch_bounds__(kBins) void offsets_small_kernel(uint32_t* __restrict__ hist, int tiles)
+{
+    __shared__ uint32_t s_wave[kBins / kWave];
+    const int d = threadIdx.x;
+    const int lane = d & (kWave - 1), wave = d / kWave;
+    uint32_t c[kSmallRows];
+#pragma unroll
+    for (int t = 0; t < kSmallRows; t++) c[t] = t < tiles ? hist[(size_t)t * kBins + d] : 0u;
+    uint32_t total = 0;
+#pragma unroll
+    for (int t = 0; t < kSmallRows; t++) total += c[t];
+    uint32_t incl = wave_inclusive_sum(total);
+    if (lane == kWave - 1) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t run = incl - total;
+    for (int w = 0; w < wave; w++) run += s_wave[w];
+#pragma unroll
+    for (int t = 0; t < kSmallRows; t++) {
+        if (t < tiles) hist[(size_t)t * kBins + d] = run;
+        run += c[t];
+    }
+}
+
 // ---- step 3: stable scatter ---------------------------------------------------------------------------
 
 __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
@@ -895,8 +922,12 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         const int shift = 32 + 8 * p;
         const int nbits = tile_bits - 8 * p < 8 ? tile_bits - 8 * p : 8;
         hipLaunchKernelGGL(count_kernel, dim3(ws.tiles), dim3(kSortBlock), 0, st, src_k, n, shift, nbits, hist);
-        hipLaunchKernelGGL(chunk_sum_kernel, dim3(ws.chunks), dim3(kBins), 0, st, hist, ws.tiles, ws.chunk, chunk_sums);
-        hipLaunchKernelGGL(offsets_kernel, dim3(ws.chunks), dim3(kBins * (ws.chunks > 16 ? kOffsetGroups : 1)), 0, st, hist, ws.tiles, ws.chunk, chunk_sums, ws.chunks);
+        if (ws.tiles <= kSmallRows) {
+            hipLaunchKernelGGL(offsets_small_kernel, dim3(1), dim3(kBins), 0, st, hist, ws.tiles);
+        } else {
+            hipLaunchKernelGGL(chunk_sum_kernel, dim3(ws.chunks), dim3(kBins), 0, st, hist, ws.tiles, ws.chunk, chunk_sums);
+            hipLaunchKernelGGL(offsets_kernel, dim3(ws.chunks), dim3(kBins * (ws.chunks > 16 ? kOffsetGroups : 1)), 0, st, hist, ws.tiles, ws.chunk, chunk_sums, ws.chunks);
+        }
         hipLaunchKernelGGL(scatter_kernel, dim3(ws.tiles), dim3(kSortBlock), 0, st,
                            src_k, src_v, dst_k, dst_v, n, shift, nbits, hist);
         src_k = dst_k;
