@@ -457,11 +457,14 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(4, 4))) v
     blend_tile<SX, SY>(FGS_BLEND_ARGS);
 }
 
-// For a frame that is resident at once, one wave per tile means that the launch lasts as long as
-// the longest list.  Here a workgroup of four waves takes four tiles that lie far apart (a long
-// list then usually has three short neighbours): every wave blends the first kOwnShare entries of
-// its own tile, and what is left of a tile after that is cut into four runs of pairs, one per
-// wave.  A run is blended from T = 1, C = 0 and the owner folds the runs in front-to-back order,
+// A frame of few tiles is placed on the chip almost at once, one wave per tile: the launch then
+// lasts as long as the busiest SIMD (the sum of the lists placed on it) and at least as long as
+// the longest list walked by one wave.  Here the tiles are ranked by list length
+// (tile_order_kernel) and a workgroup of four waves takes one tile from each quarter of the
+// ranking: the workgroups with the longest lists are dispatched first, the short ones fill in
+// behind them, and a long list has three shorter ones beside it.  Every wave blends the first
+// kOwnShare entries of its own tile; what is left of a list of more than kOwnShare + kMinRest
+// entries after that is cut into four runs of pairs, one per wave.  A run is blended from T = 1, C = 0 and the owner folds the runs in front-to-back order,
 // C += T C_run, T *= T_run, which is the same sum in another order of additions.  A run stops
 // when its own T is below the threshold everywhere, so a tile can be walked a little further than
 // the reference walks it: what that adds is below 1e-4 of a colour.
