@@ -13,7 +13,8 @@
 //    end to end and tested one per lane per step, so lanes stay busy whatever the mix of sizes;
 //    larger rectangles are tested by the whole wave, 64 tiles a step, and rectangles of more than
 //    1024 tiles by the whole workgroup, which gets the passing tiles of every column and row as
-//    an interval found by bisection with the reference's own edge predicates.
+//    an interval found by bisection with the reference's own edge predicates: the tiles are
+//    counted from the intervals alone and visited only to write their keys.
 //
 // THIS FILE MUST BE COMPILED WITH -ffp-contract=off.  Every fp32 expression that feeds a key is
 // written in the operand order of the reference and has to be evaluated one IEEE operation at a
@@ -29,7 +30,10 @@ constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kStashCap = 1024;         // flat candidates (and so stashed hits) per wave
 constexpr int kHugeMin = 1024;          // rectangles with more tiles than this are tested by the whole workgroup
-constexpr int kHugeCap = 16;            // such rectangles per workgroup; further ones stay with their wave
+// such rectangles per workgroup: as many as the LDS of 7 workgroups per CU leaves room for (a
+// rectangle beyond the list stays with its wave, 64 tiles a step, and everything behind this
+// workgroup in the chained scan waits for that count)
+constexpr int kHugeCap = 27;
 constexpr int kSpanWords = kWavesPerBlock * kStashCap / 4;   // column + row spans of one listed rectangle
 static_assert(kSpanWords / kWave <= kWave, "one lane per group of 64 columns");
 constexpr unsigned kSpinLimit = 1u << 22;   // polls before a chained-scan wait gives up
@@ -204,20 +208,18 @@ __device__ __forceinline__ uint32_t edge_span(float a, float cony, float c_acros
     const uint32_t inside = (centre >= (float)lo_px && centre <= (float)hi_px) ? 1u << 30 : 0u;
     const EdgeTest e = edge_test(a, cony, c_across, centre, lo_px, hi_px, w);
     if (!(e.delta >= 0.0f)) return inside | 1u;
-    int lo = 0, hi = count;             // near_ok holds for tiles [0, lo), fails from hi on
-    while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (near_ok(e, (float)((first_tile_along + mid) * block_along), centre_along)) lo = mid + 1;
-        else hi = mid;
+    // Two bisections side by side, so that their dependent chains overlap: near_ok holds for
+    // tiles [0, n_lo) and fails from n_hi on; far_ok fails for tiles [0, f_lo), holds from f_hi on.
+    int n_lo = 0, n_hi = count, f_lo = 0, f_hi = count;
+    while (n_lo < n_hi || f_lo < f_hi) {
+        const int n_mid = (n_lo + n_hi) >> 1, f_mid = (f_lo + f_hi) >> 1;
+        const bool n_ok = near_ok(e, (float)((first_tile_along + n_mid) * block_along), centre_along);
+        const bool f_ok = far_ok(e, (float)((first_tile_along + f_mid) * block_along + block_along - 1), centre_along);
+        if (n_lo < n_hi) { if (n_ok) n_lo = n_mid + 1; else n_hi = n_mid; }
+        if (f_lo < f_hi) { if (f_ok) f_hi = f_mid; else f_lo = f_mid + 1; }
     }
-    const int last = lo - 1;
-    lo = 0; hi = count;                 // far_ok fails for tiles [0, lo), holds from hi on
-    while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (far_ok(e, (float)((first_tile_along + mid) * block_along + block_along - 1), centre_along)) hi = mid;
-        else lo = mid + 1;
-    }
-    const int first = lo;
+    const int last = n_lo - 1;
+    const int first = f_lo;
     if (first > last) return inside | 1u;
     return inside | (uint32_t)first | ((uint32_t)last << 15);
 }
@@ -417,6 +419,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     __shared__ uint32_t s_huge_cnt[kHugeCap][kWavesPerBlock];
     __shared__ int s_huge_spans[kHugeCap];                      // 1: the tiles that pass are found from column and row spans
     __shared__ int s_nhuge;
+    __shared__ int s_centre[2];                                 // column and row of a listed rectangle that hold its centre
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -687,11 +690,61 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
             }
         }
     };
+    // How many tiles of listed rectangle e pass, per quarter of its rows (the quarters are the
+    // waves' shares when the keys are written).  From the spans no tile has to be visited: a tile
+    // passes if its row's span holds its column, or its column's span holds its row, or it is
+    // the tile of the centre.  The rows add up their spans; every column goes down its own span
+    // and counts the rows whose span does not hold it already.
+    auto count_from_spans = [&](int e) {
+        const int grw = s_huge_i[e][2];
+        const int grh = s_huge_i[e][3] / grw;
+        const int rows = (grh + kWavesPerBlock - 1) / kWavesPerBlock;
+        auto add = [&](int ty, uint32_t v) {
+            int q = 0;
+#pragma unroll
+            for (int k = 1; k < kWavesPerBlock; k++) q += ty >= k * rows ? 1 : 0;
+            atomicAdd(&s_huge_cnt[e][q], v);
+        };
+        for (int ty = tid; ty < grh; ty += kBlock) {
+            const uint32_t row = spans[grw + ty];
+            const uint32_t rlo = row & 0x7fffu, rhi = (row >> 15) & 0x7fffu;
+            if (rlo <= rhi) add(ty, rhi - rlo + 1u);
+            if (row >> 30) s_centre[1] = ty;
+        }
+        for (int tx = tid; tx < grw; tx += kBlock) {
+            const uint32_t col = spans[tx];
+            const uint32_t clo = col & 0x7fffu, chi = (col >> 15) & 0x7fffu;
+            if (col >> 30) s_centre[0] = tx;
+            for (uint32_t ty = clo; ty <= chi; ty++) {          // an empty span is 1 .. 0
+                const uint32_t row = spans[grw + (int)ty];
+                const uint32_t rlo = row & 0x7fffu, rhi = (row >> 15) & 0x7fffu;
+                if (!(rlo <= rhi && (uint32_t)tx >= rlo && (uint32_t)tx <= rhi)) add((int)ty, 1u);
+            }
+        }
+        __syncthreads();
+        if (tid == 0 && s_centre[0] >= 0 && s_centre[1] >= 0) {
+            // the tile of the centre, unless a span has counted it
+            const int tx = s_centre[0], ty = s_centre[1];
+            const uint32_t col = spans[tx], row = spans[grw + ty];
+            const bool by_column = (uint32_t)ty >= (col & 0x7fffu) && (uint32_t)ty <= ((col >> 15) & 0x7fffu);
+            const bool by_row = (uint32_t)tx >= (row & 0x7fffu) && (uint32_t)tx <= ((row >> 15) & 0x7fffu);
+            if (!by_column && !by_row) {
+                int q = 0;
+                while (ty >= (q + 1) * rows) q++;
+                atomicAdd(&s_huge_cnt[e][q], 1u);
+            }
+        }
+    };
     for (int e = 0; e < n_huge; e++) {
-        const bool from_spans = s_huge_spans[e] != 0;
-        if (from_spans) fill_spans(e);
+        if (s_huge_spans[e] != 0) {
+            if (tid < kWavesPerBlock) s_huge_cnt[e][tid] = 0;
+            if (tid == 0) { s_centre[0] = -1; s_centre[1] = -1; }
+            fill_spans(e);
+            count_from_spans(e);
+            continue;
+        }
         uint32_t total = 0;
-        walk_listed(e, from_spans, [&](int, int, bool ok) { total += (uint32_t)__popcll(ballot(ok)); });
+        walk_listed(e, false, [&](int, int, bool ok) { total += (uint32_t)__popcll(ballot(ok)); });
         if (lane == 0) s_huge_cnt[e][wave] = total;
     }
     if (n_huge > 0) {
