@@ -24,15 +24,16 @@ class SceneOnDevice:
         self.cov3d = dev(scene.cov3d)
 
 
-def preprocess(sd, cam, capacity, block=(16, 16), sentinel=None, start_offset=0, guard=True):
-    """Returns dict of torch tensors + num_rendered (after a sync)."""
+def preprocess(sd, cam, capacity, block=(16, 16), sentinel=None, start_offset=0, guard=True, pad=0):
+    """Returns dict of torch tensors + num_rendered (after a sync).  The key and value buffers are
+    allocated with `pad` entries beyond the capacity the library is told about."""
     n = sd.n
     fillv = 0.0 if sentinel is None else sentinel
     points_xy = torch.full((n, 2), fillv, device=DEV, dtype=torch.float32)
     rgb_depth = torch.full((n, 4), fillv, device=DEV, dtype=torch.float32)
     conic_opacity = torch.full((n, 4), fillv, device=DEV, dtype=torch.float32)
-    keys = torch.zeros(capacity, device=DEV, dtype=torch.int64)
-    values = torch.zeros(capacity, device=DEV, dtype=torch.int32)
+    keys = torch.zeros(capacity + pad, device=DEV, dtype=torch.int64)
+    values = torch.zeros(capacity + pad, device=DEV, dtype=torch.int32)
     curr_offset = torch.full((1,), start_offset, device=DEV, dtype=torch.int32)
     cabi.preprocess(n, sd.position.data_ptr(), sd.shs.data_ptr(), sd.opacity.data_ptr(), sd.cov3d.data_ptr(),
                     cam.width, cam.height, block[0], block[1], cam.position, cam.rotation,

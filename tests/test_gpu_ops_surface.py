@@ -85,3 +85,68 @@ def test_ops_errors_on_the_gpu():
         fgs.ops.render_16x16(K, cam.width, cam.height, rast.points_xy, rast.rgb_depth, rast.conic_opacity,
                              rast.gaussian_keys_sorted, rast.gaussian_values_sorted, rast.ranges[:10], torch.zeros(3),
                              torch.zeros((cam.height, cam.width, 3), device="cuda:0", dtype=torch.uint8))
+
+
+def _write_ply(path, recs):
+    props = ["x", "y", "z", "nx", "ny", "nz"] + ["f_dc_%d" % i for i in range(3)] + ["f_rest_%d" % i for i in range(45)] \
+        + ["opacity"] + ["scale_%d" % i for i in range(3)] + ["rot_%d" % i for i in range(4)]
+    head = "ply\nformat binary_little_endian 1.0\nelement vertex %d\n" % len(recs)
+    head += "".join("property float %s\n" % p for p in props) + "end_header\n"
+    with open(path, "wb") as fh:
+        fh.write(head.encode())
+        fh.write(np.ascontiguousarray(recs, dtype="<f4").tobytes())
+
+
+def test_render_scene_from_ply_and_cameras_json(oracle, tmp_path, capsys):
+    """The file path of example.py:105-144: a 3DGS model directory (point_cloud.ply of 62-float
+    records + cameras.json) goes through loadPly -> device -> preprocess -> sort -> render -> .ppm,
+    and every image is the oracle's image of the same Gaussians (those loadPly returns)."""
+    import json
+    import flash_gaussian_splatting as fgs
+    from flashgs_amd.rasterizer import render_scene
+    rng = np.random.default_rng(21)
+    n = 30_000
+    recs = np.zeros((n, 62), np.float32)
+    recs[:, 0:3] = rng.uniform(-5.0, 5.0, (n, 3))
+    recs[:, 3:6] = rng.standard_normal((n, 3))                   # normals: ignored by the loader
+    recs[:, 6:9] = 0.5 * rng.standard_normal((n, 3))             # f_dc
+    recs[:, 9:54] = 0.05 * rng.standard_normal((n, 45))          # f_rest, planar
+    recs[:, 54] = 1.5 * rng.standard_normal(n)                   # opacity logit
+    recs[:, 55:58] = -3.2 + 0.6 * rng.standard_normal((n, 3))    # log-scales
+    recs[:, 58:62] = rng.standard_normal((n, 4)) * 3.0           # quaternion, not normalised
+    model = tmp_path / "model"
+    ply_dir = model / "point_cloud" / "iteration_30000"
+    ply_dir.mkdir(parents=True)
+    _write_ply(str(ply_dir / "point_cloud.ply"), recs)
+    cams = []
+    for k, (w, h, pos) in enumerate([(1280, 720, [0.0, 0.0, -15.0]), (1000, 600, [1.0, -0.5, -13.0])]):
+        c = scenes.look_at(pos, [0, 0, 0], w, h, 50.0)
+        cams.append(dict(id=k, img_name="view_%d" % k, width=w, height=h, position=[float(v) for v in c.position],
+                         rotation=[[float(v) for v in row] for row in c.rotation], fx=c.focal_x, fy=c.focal_y))
+    (model / "cameras.json").write_text(json.dumps(cams))
+
+    render_scene(str(model), test_performance=True, MAX_NUM_RENDERED=1 << 20, MAX_NUM_TILES=1 << 13)
+    out = capsys.readouterr().out
+    assert "num_vertex = %d" % n in out and "fps = " in out
+
+    num, position, shs, opacity, cov3d = fgs.ops.loadPly(str(ply_dir / "point_cloud.ply"))
+    assert num == n
+    for cj in cams:
+        w, h = cj["width"], cj["height"]
+        pos = np.array(cj["position"], np.float32)
+        rot = np.array(cj["rotation"], np.float32)
+        pre = oracle.preprocess(position.numpy(), shs.numpy(), opacity.numpy(), cov3d.numpy(), w, h, 16, 16, pos, rot,
+                                cj["fx"], cj["fy"], 100.0, 0.01, 1 << 20)
+        K = pre["num_rendered"]
+        assert K > 10_000
+        ks, vs = oracle.sort(K, w, h, 16, 16, pre["keys"], pre["values"])
+        rg = oracle.ranges(K, ks, ((w + 15) // 16) * ((h + 15) // 16))
+        u8, _, _ = oracle.render(w, h, 16, 16, pre["points_xy"], pre["rgb_depth"], pre["conic_opacity"], vs, rg,
+                                 np.zeros(3, np.float32), want_f32=False)
+        data = (model / "test_out" / ("%s.ppm" % cj["img_name"])).read_bytes()
+        head = b"P6\n%d %d\n255\n" % (w, h)
+        assert data.startswith(head) and len(data) == len(head) + 3 * w * h
+        img = np.frombuffer(data[len(head):], np.uint8).reshape(h, w, 3)
+        d = np.abs(img.astype(np.int16) - u8.astype(np.int16))
+        assert d.max() <= 1 and (d > 0).mean() < 0.01
+        assert img.max() > 100          # not an empty frame

@@ -479,6 +479,52 @@ def test_full_size_configs(oracle, config):
             assert ref["pre"]["counts"]["candidates"] > 3 * ref["K"]
 
 
+def test_orbit_config_at_4k(oracle):
+    """The 2M orbit at 3840x2160, first, middle and last pose: the needles next to the camera have
+    candidate rectangles of thousands of tiles, which the workgroup tests from column and row spans."""
+    sc = scenes.make(4, width=3840, height=2160)
+    for cam in (sc.cameras[0], sc.cameras[len(sc.cameras) // 2], sc.cameras[-1]):
+        ref = _check_frame(oracle, sc, cam, 1 << 25)
+        assert ref["pre"]["counts"]["candidates"] > 5 * ref["K"]
+
+
+@pytest.fixture(scope="module")
+def config3_scene():
+    return scenes.make(3)
+
+
+def test_config3_8k_frame(oracle, config3_scene):
+    """8M Gaussians at 7680x4320 (129 600 tiles, three partition passes, the blend variant with
+    fewer resident waves), 2 % of the splats enlarged: the whole frame against the oracle."""
+    sc = config3_scene
+    ref = _check_frame(oracle, sc, sc.cameras[0], 1 << 25)
+    assert ref["K"] > 10_000_000
+
+
+def test_config3_more_than_100M_pairs(oracle, config3_scene):
+    """The same scene with every splat five times as large: more than 100M pairs in a key buffer of
+    2^27 entries (example.py:123), slot arithmetic far beyond 2^24, hundreds of tiles with more
+    than 8192 pairs.  The whole frame against the oracle; then with a key buffer smaller than the
+    pair count: the count is still the full one and nothing is written past the capacity
+    (the reference would write out of bounds there, preprocess.cu:330,395; example.py:79-82 only
+    checks afterwards)."""
+    import copy
+    import gpu_pipeline as gp
+    sc = copy.copy(config3_scene)
+    sc.cov3d = (config3_scene.cov3d * np.float32(25.0)).astype(np.float32)
+    cam = sc.cameras[0]
+    ref = _check_frame(oracle, sc, cam, 1 << 27)
+    K = ref["K"]
+    assert K > 100_000_000
+    assert ((ref["ranges"][:, 1] - ref["ranges"][:, 0]) > 8192).sum() > 100
+    cap = 100_000_000
+    got = gp.preprocess(gp.SceneOnDevice(sc), cam, cap, pad=1 << 20)
+    assert got["num_rendered"] == K
+    assert np.array_equal(gp.u64(got["keys"])[:cap], ref["pre"]["keys"][:cap])
+    assert np.array_equal(gp.u32(got["values"])[:cap], ref["pre"]["values"][:cap])
+    assert not gp.u64(got["keys"])[cap:].any() and not gp.u32(got["values"])[cap:].any()
+
+
 def _sort_case(tile, depth_bits, W, H, junk=None, seed=0):
     import gpu_pipeline as gp
     rng = np.random.default_rng(seed)
