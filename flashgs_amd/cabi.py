@@ -20,6 +20,8 @@ _RENDER_ARGS = [C.c_int] * 3 + [C.c_void_p] * 8 + [C.c_void_p]
 SIGNATURES = {
     "fgs_preprocess": (C.c_int, [C.c_int] + [C.c_void_p] * 4 + [C.c_int] * 4 + [C.c_void_p] * 2 + [C.c_float] * 4
                        + [C.c_void_p] * 6 + [C.c_int64, C.c_void_p]),
+    "fgs_preprocess_static": (C.c_int, [C.c_int] + [C.c_void_p] * 4 + [C.c_int] * 4 + [C.c_void_p] * 2 + [C.c_float] * 4
+                              + [C.c_void_p] * 6 + [C.c_int64, C.c_void_p]),
     "fgs_sort_gaussian": (C.c_int, [C.c_int] * 5 + [C.c_void_p, C.c_size_t] + [C.c_void_p] * 4 + [C.c_void_p]),
     "fgs_get_sort_buffer_size": (C.c_size_t, [C.c_int]),
     "fgs_render_16x16": (C.c_int, _RENDER_ARGS),
@@ -78,13 +80,15 @@ def camera_matrices(position, rotation, width, height, focal_x, focal_y, zFar, z
 
 def preprocess(P, positions, shs, opacities, cov3ds, width, height, block_x, block_y, position, rotation,
                focal_x, focal_y, zFar, zNear, points_xy, rgb_depth, conic_opacity, keys, values, curr_offset,
-               key_capacity=0, stream=0):
+               key_capacity=0, stream=0, static=False):
+    """``static=True`` calls fgs_preprocess_static, the variant that allocates nothing."""
     pos, rot = _host_f32(position, 3), _host_f32(rotation, 9)
-    rc = load().fgs_preprocess(P, positions, shs, opacities, cov3ds, width, height, block_x, block_y,
+    fn = load().fgs_preprocess_static if static else load().fgs_preprocess
+    rc = fn(P, positions, shs, opacities, cov3ds, width, height, block_x, block_y,
                                pos.ctypes.data, rot.ctypes.data, focal_x, focal_y, zFar, zNear,
                                points_xy, rgb_depth, conic_opacity, keys, values, curr_offset,
-                               key_capacity, stream)
-    _check(rc, "fgs_preprocess")
+            key_capacity, stream)
+    _check(rc, "fgs_preprocess_static" if static else "fgs_preprocess")
 
 
 def get_sort_buffer_size(num_rendered):

@@ -401,7 +401,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     uint32_t* __restrict__ values,
     int* __restrict__ curr_offset,
     int64_t capacity,            // <= 0: unchecked
-    uint64_t* __restrict__ scratch,        // control word, then two status arrays of status_capacity words
+    uint64_t* __restrict__ scan_words,     // control word, then two status arrays of status_capacity words
     int status_capacity,
     int num_blocks)
 {
@@ -433,10 +433,10 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     const int ticket = (int)blockIdx.x;
     const int idx = ticket * kBlock + tid;
     // this launch's status array; the other one is cleared for the launch that follows
-    const uint32_t which = (uint32_t)peek(scratch) & 1u;
-    uint64_t* const status = scratch + kControlWords + (size_t)which * status_capacity;
+    const uint32_t which = (uint32_t)peek(scan_words) & 1u;
+    uint64_t* const status = scan_words + kControlWords + (size_t)which * status_capacity;
     {
-        uint64_t* const other = scratch + kControlWords + (size_t)(which ^ 1u) * status_capacity;
+        uint64_t* const other = scan_words + kControlWords + (size_t)(which ^ 1u) * status_capacity;
         for (long long w = ticket + (long long)tid * num_blocks; w < status_capacity; w += (long long)kBlock * num_blocks)
             other[w] = 0;
     }
@@ -796,7 +796,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
             // and hands the other status array to the next launch
             if (ticket == num_blocks - 1) {
                 *curr_offset = timed_out ? -2147483647 - 1 : (int)(excl + block_total);
-                publish(scratch, (uint64_t)(which ^ 1u));
+                publish(scan_words, (uint64_t)(which ^ 1u));
             }
         }
     }
@@ -964,31 +964,59 @@ extern "C" void fgs_camera_matrices(const float cam_position[3], const float cam
     fgs::camera_matrices(cam_position, cam_rotation, width, height, focal_x, focal_y, zFar, zNear, view, proj);
 }
 
-extern "C" int fgs_preprocess(int P,
-                              const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
-                              int width, int height, int block_x, int block_y,
-                              const float cam_position[3], const float cam_rotation[9],
-                              float focal_x, float focal_y, float zFar, float zNear,
-                              float* points_xy, float* rgb_depth, float* conic_opacity,
-                              uint64_t* gaussian_keys_unsorted, uint32_t* gaussian_values_unsorted,
-                              int* curr_offset, int64_t key_capacity, void* stream)
+namespace fgs {
+namespace {
+
+// ---- scan status held in the library's own image, for callers that cannot allocate ----------------
+//
+// The same two status arrays as the allocated scratch, as a file-scope device array: one copy per
+// GPU that loads the library, zero when the code object is loaded, kept until the process ends.
+// In host code the array's name is only a handle; the device address comes from
+// hipGetSymbolAddress, once per device with that device current.
+constexpr int kStaticBlocks = 1 << 16;                        // workgroups one status array holds
+constexpr int kStaticMaxP = kStaticBlocks * kBlock;           // 16 777 216 Gaussians
+static __device__ __align__(256) uint64_t scratch[kControlWords + 2 * kStaticBlocks];
+uint64_t* g_static_words[kMaxDevices];                        // device address of `scratch`, per device
+
+int static_scratch(int device, uint64_t** out)
 {
-    using namespace fgs;
-    if (P < 0) return fail(FGS_E_INVALID, "fgs_preprocess: P = %d is negative", P);
+    if (!g_static_words[device]) {
+        void* ptr = nullptr;
+        FGS_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return fail(FGS_E_HIP, "hipGetSymbolAddress returned a null address for the scan status");
+        g_static_words[device] = (uint64_t*)ptr;
+    }
+    *out = g_static_words[device];
+    return FGS_OK;
+}
+
+int preprocess_impl(bool allocate, const char* who, int P,
+                    const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
+                    int width, int height, int block_x, int block_y,
+                    const float cam_position[3], const float cam_rotation[9],
+                    float focal_x, float focal_y, float zFar, float zNear,
+                    float* points_xy, float* rgb_depth, float* conic_opacity,
+                    uint64_t* gaussian_keys_unsorted, uint32_t* gaussian_values_unsorted,
+                    int* curr_offset, int64_t key_capacity, void* stream)
+{
+    if (P < 0) return fail(FGS_E_INVALID, "%s: P = %d is negative", who, P);
     if (width <= 0 || height <= 0 || block_x <= 0 || block_y <= 0)
-        return fail(FGS_E_INVALID, "fgs_preprocess: width/height/block must be positive (got %d x %d, block %d x %d)",
-                    width, height, block_x, block_y);
-    if (!cam_position || !cam_rotation) return fail(FGS_E_INVALID, "fgs_preprocess: null camera");
-    if (!curr_offset) return fail(FGS_E_INVALID, "fgs_preprocess: null curr_offset");
+        return fail(FGS_E_INVALID, "%s: width/height/block must be positive (got %d x %d, block %d x %d)",
+                    who, width, height, block_x, block_y);
+    if (!cam_position || !cam_rotation) return fail(FGS_E_INVALID, "%s: null camera", who);
+    if (!curr_offset) return fail(FGS_E_INVALID, "%s: null curr_offset", who);
     if (P > 0 && (!positions || !shs || !opacities || !cov3Ds || !points_xy || !rgb_depth || !conic_opacity ||
                   !gaussian_keys_unsorted || !gaussian_values_unsorted))
-        return fail(FGS_E_INVALID, "fgs_preprocess: null buffer");
+        return fail(FGS_E_INVALID, "%s: null buffer", who);
+    if (!allocate && P > kStaticMaxP)
+        return fail(FGS_E_INVALID, "%s: P = %d exceeds the %d Gaussians the built-in scan status holds "
+                                   "(fgs_preprocess has no such limit)", who, P, kStaticMaxP);
     if (P == 0) return FGS_OK;
     if (((uintptr_t)shs | (uintptr_t)rgb_depth | (uintptr_t)conic_opacity) % 16 != 0 ||
         ((uintptr_t)cov3Ds | (uintptr_t)points_xy | (uintptr_t)gaussian_keys_unsorted) % 8 != 0)
-        return fail(FGS_E_INVALID, "fgs_preprocess: shs/rgb_depth/conic_opacity must be 16-byte aligned, "
-                                   "cov3Ds/points_xy/keys 8-byte aligned");
-    if ((long long)P + kBlock > 2147483647LL) return fail(FGS_E_INVALID, "fgs_preprocess: P = %d too large", P);
+        return fail(FGS_E_INVALID, "%s: shs/rgb_depth/conic_opacity must be 16-byte aligned, "
+                                   "cov3Ds/points_xy/keys 8-byte aligned", who);
+    if ((long long)P + kBlock > 2147483647LL) return fail(FGS_E_INVALID, "%s: P = %d too large", who, P);
 
     Camera cam;
     camera_matrices(cam_position, cam_rotation, width, height, focal_x, focal_y, zFar, zNear, cam.view, cam.proj);
@@ -1002,18 +1030,61 @@ extern "C" int fgs_preprocess(int P,
 
     int device = 0;
     FGS_HIP_TRY(hipGetDevice(&device));
-    if (device < 0 || device >= kMaxDevices) return fail(FGS_E_INVALID, "fgs_preprocess: device %d unsupported", device);
+    if (device < 0 || device >= kMaxDevices) return fail(FGS_E_INVALID, "%s: device %d unsupported", who, device);
     const int num_blocks = (P + kBlock - 1) / kBlock;
     hipStream_t st = (hipStream_t)stream;
 
     std::lock_guard<std::mutex> lock(g_mutex);
-    Scratch* s = nullptr;
-    int rc = acquire_scratch(device, num_blocks, st, &s);
-    if (rc != FGS_OK) return rc;
+    uint64_t* words = nullptr;
+    int status_capacity = 0;
+    if (allocate) {
+        Scratch* s = nullptr;
+        int rc = acquire_scratch(device, num_blocks, st, &s);
+        if (rc != FGS_OK) return rc;
+        words = s->words;
+        status_capacity = (int)s->capacity;
+    } else {
+        int rc = static_scratch(device, &words);
+        if (rc != FGS_OK) return rc;
+        status_capacity = kStaticBlocks;
+    }
 
     hipLaunchKernelGGL(preprocess_kernel, dim3(num_blocks), dim3(kBlock), 0, st,
                        P, positions, shs, opacities, cov3Ds, cam, points_xy, rgb_depth, conic_opacity,
                        gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset, key_capacity,
-                       s->words, (int)s->capacity, num_blocks);
+                       words, status_capacity, num_blocks);
     return check_hip(hipGetLastError(), "preprocess_kernel launch");
+}
+
+} // namespace
+} // namespace fgs
+
+extern "C" int fgs_preprocess(int P,
+                              const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
+                              int width, int height, int block_x, int block_y,
+                              const float cam_position[3], const float cam_rotation[9],
+                              float focal_x, float focal_y, float zFar, float zNear,
+                              float* points_xy, float* rgb_depth, float* conic_opacity,
+                              uint64_t* gaussian_keys_unsorted, uint32_t* gaussian_values_unsorted,
+                              int* curr_offset, int64_t key_capacity, void* stream)
+{
+    return fgs::preprocess_impl(true, "fgs_preprocess", P, positions, shs, opacities, cov3Ds, width, height, block_x, block_y,
+                                cam_position, cam_rotation, focal_x, focal_y, zFar, zNear, points_xy, rgb_depth,
+                                conic_opacity, gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset,
+                                key_capacity, stream);
+}
+
+extern "C" int fgs_preprocess_static(int P,
+                                     const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
+                                     int width, int height, int block_x, int block_y,
+                                     const float cam_position[3], const float cam_rotation[9],
+                                     float focal_x, float focal_y, float zFar, float zNear,
+                                     float* points_xy, float* rgb_depth, float* conic_opacity,
+                                     uint64_t* gaussian_keys_unsorted, uint32_t* gaussian_values_unsorted,
+                                     int* curr_offset, int64_t key_capacity, void* stream)
+{
+    return fgs::preprocess_impl(false, "fgs_preprocess_static", P, positions, shs, opacities, cov3Ds, width, height,
+                                block_x, block_y, cam_position, cam_rotation, focal_x, focal_y, zFar, zNear, points_xy,
+                                rgb_depth, conic_opacity, gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset,
+                                key_capacity, stream);
 }

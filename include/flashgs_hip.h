@@ -63,6 +63,25 @@ int fgs_preprocess(int P,
                    int* curr_offset, int64_t key_capacity, void* stream);
 
 /*
+ * No counterpart in the reference.  fgs_preprocess for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * same arguments, same kernel, same results, but the scan status lives in a 1 MiB array inside
+ * the library's device image (one copy per GPU, held until the process ends) instead of a
+ * buffer from hipMalloc, so the call allocates and frees nothing and never synchronises.
+ * P is limited to 16 777 216 Gaussians; a larger P returns FGS_E_INVALID.  Every call on one GPU
+ * shares that GPU's array: calls that overlap in time on one GPU race (calls on one stream, or
+ * otherwise ordered, do not).  May be mixed freely with fgs_preprocess.
+ */
+int fgs_preprocess_static(int P,
+                          const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
+                          int width, int height, int block_x, int block_y,
+                          const float cam_position[3], const float cam_rotation[9],
+                          float focal_x, float focal_y, float zFar, float zNear,
+                          float* points_xy, float* rgb_depth, float* conic_opacity,
+                          uint64_t* gaussian_keys_unsorted, uint32_t* gaussian_values_unsorted,
+                          int* curr_offset, int64_t key_capacity, void* stream);
+
+/*
  * Replaces flashgs::sort_gaussian (csrc/ops.h:41-45, csrc/cuda_rasterizer/sort.cu:28-44):
  * stable ascending sort of num_rendered (key, value) pairs on key bits
  * [0, 32 + bit_length(tiles_x * tiles_y)).  Inputs are left untouched.

@@ -24,7 +24,7 @@ class SceneOnDevice:
         self.cov3d = dev(scene.cov3d)
 
 
-def preprocess(sd, cam, capacity, block=(16, 16), sentinel=None, start_offset=0, guard=True, pad=0):
+def preprocess(sd, cam, capacity, block=(16, 16), sentinel=None, start_offset=0, guard=True, pad=0, static=False):
     """Returns dict of torch tensors + num_rendered (after a sync).  The key and value buffers are
     allocated with `pad` entries beyond the capacity the library is told about."""
     n = sd.n
@@ -40,7 +40,7 @@ def preprocess(sd, cam, capacity, block=(16, 16), sentinel=None, start_offset=0,
                     cam.focal_x, cam.focal_y, cam.zFar, cam.zNear,
                     points_xy.data_ptr(), rgb_depth.data_ptr(), conic_opacity.data_ptr(),
                     keys.data_ptr(), values.data_ptr(), curr_offset.data_ptr(),
-                    capacity if guard else 0, torch.cuda.current_stream().cuda_stream)
+                    capacity if guard else 0, torch.cuda.current_stream().cuda_stream, static=static)
     num = int(curr_offset.cpu()[0])
     return dict(points_xy=points_xy, rgb_depth=rgb_depth, conic_opacity=conic_opacity, keys=keys, values=values,
                 num_rendered=num)
