@@ -31,6 +31,7 @@ SIGNATURES = {
     "fgs_tile_ranges": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 3),
     "fgs_blend": (C.c_int, [C.c_int] * 4 + [C.c_void_p] * 9),
     "fgs_camera_matrices": (None, [C.c_void_p] * 2 + [C.c_int] * 2 + [C.c_float] * 4 + [C.c_void_p] * 2),
+    "fgs_set_scan_spin_limit": (C.c_uint, [C.c_uint]),
     "fgs_last_error": (C.c_char_p, []),
     "fgs_abi_version": (C.c_int, []),
 }
@@ -89,6 +90,11 @@ def preprocess(P, positions, shs, opacities, cov3ds, width, height, block_x, blo
                                points_xy, rgb_depth, conic_opacity, keys, values, curr_offset,
             key_capacity, stream)
     _check(rc, "fgs_preprocess_static" if static else "fgs_preprocess")
+
+
+def set_scan_spin_limit(polls):
+    """Polls after which a wait inside the preprocess launch gives up; returns the previous value."""
+    return int(load().fgs_set_scan_spin_limit(polls))
 
 
 def get_sort_buffer_size(num_rendered):

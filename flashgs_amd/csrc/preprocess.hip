@@ -6,9 +6,10 @@
 // key - SH colour and the 40-byte attribute record.
 //
 // Differences in mechanism (not in results):
-//  * Key slots come from a count -> wave scan -> block scan -> chained look-back over
-//    workgroups instead of atomics on one counter, so the unsorted list has a fixed order:
-//    ascending Gaussian index, then row-major tiles.  A stable sort then fixes tie order too.
+//  * Key slots come from a count -> wave scan -> block scan -> scan over workgroups by one
+//    dedicated wave of the launch instead of atomics on one counter, so the unsorted list has a
+//    fixed order: ascending Gaussian index, then row-major tiles.  A stable sort then fixes tie
+//    order too.
 //  * The candidate tiles of all Gaussians of a wave with rectangles of at most 64 tiles are laid
 //    end to end and tested one per lane per step, so lanes stay busy whatever the mix of sizes;
 //    larger rectangles are tested by the whole wave, 64 tiles a step, and rectangles of more than
@@ -21,6 +22,7 @@
 // time, so that a scalar CPU evaluation of the same expressions gives the same bits.
 #include "fgs_internal.h"
 
+#include <atomic>
 #include <mutex>
 
 namespace fgs {
@@ -32,11 +34,11 @@ constexpr int kStashCap = 1024;         // flat candidates (and so stashed hits)
 constexpr int kHugeMin = 1024;          // rectangles with more tiles than this are tested by the whole workgroup
 // such rectangles per workgroup: as many as the LDS of 7 workgroups per CU leaves room for (a
 // rectangle beyond the list stays with its wave, 64 tiles a step, and everything behind this
-// workgroup in the chained scan waits for that count)
+// workgroup waits for that count)
 constexpr int kHugeCap = 27;
 constexpr int kSpanWords = kWavesPerBlock * kStashCap / 4;   // column + row spans of one listed rectangle
 static_assert(kSpanWords / kWave <= kWave, "one lane per group of 64 columns");
-constexpr unsigned kSpinLimit = 1u << 22;   // polls before a chained-scan wait gives up
+constexpr unsigned kSpinLimit = 1u << 22;   // polls before a wait on the scan over workgroups gives up
 
 struct Camera {
     float view[16];
@@ -304,20 +306,34 @@ __device__ __forceinline__ void sh_to_rgb(const float* __restrict__ sh, float px
     }
 }
 
-// ---- chained scan over workgroups ---------------------------------------------------------------
+// ---- scan over workgroups ------------------------------------------------------------------------
 //
-// status word: [33:32] state, [31:0] count; 0 = nothing published yet.
-// The scratch holds a control word and two status arrays.  A launch works in the array the
-// control word names and clears the other one, which the launch after it will use; its last
-// workgroup flips the control word when its own walk back is over.  That walk ends only when
-// every earlier workgroup has published, i.e. after all of them have read the control word, so
-// no workgroup of this launch can see the flipped value; the next launch (same stream, or
-// otherwise ordered after this one) starts from it.  Nothing on the host changes from launch to
-// launch, so a captured launch can be replayed.
-constexpr int kControlWords = 8;          // control word + padding in front of the two arrays
-constexpr uint64_t kStateAggregate = 1;   // count of this workgroup only
-constexpr uint64_t kStatePrefix = 2;      // count of this workgroup and all before it
-constexpr uint64_t kStatePoison = 3;      // like kStatePrefix, but a predecessor never published
+// Key slots are handed out in workgroup order.  Every workgroup publishes its key count as soon
+// as it knows it; one wave of the launch (the scanner: the first wave of workgroup 0, which does
+// nothing else) reads the counts in order, 128 per trip to memory, and publishes for every
+// workgroup the number of keys in front of it; a workgroup picks that number up after its colour
+// work, when it has long been written.  Nobody but the scanner reads other workgroups' counts, so
+// the wait of a workgroup is one read of one word, whatever else loads the memory system.
+//
+// status word: [33:32] state, [31:0] value; 0 = nothing published yet.
+// The scan words hold a control word and two generations of (counts, offsets) arrays.  A launch
+// works in the generation the control word names and clears the other one, which the launch
+// after it will use; the scanner flips the control word when it has read the last count, i.e.
+// after every workgroup of this launch has read the control word, so no workgroup of this launch
+// can see the flipped value; the next launch (same stream, or otherwise ordered after this one)
+// starts from it.  Nothing on the host changes from launch to launch, so a captured launch can be
+// replayed.
+//
+// Every wait is bounded by spin_limit polls.  A wait that gives up makes the launch report a
+// negative pair count: the scanner marks all offsets it can no longer compute as poisoned, a
+// workgroup that gave up on its offset (or found it poisoned) writes its keys from slot 0 and
+// lowers *curr_offset to INT_MIN, and the scanner's own final write of the total is a
+// compare-and-swap against the starting value, so INT_MIN stays whichever comes first.
+constexpr int kControlWords = 8;          // control word + padding in front of the arrays
+constexpr uint64_t kStateCount = 1;       // key count of one workgroup
+constexpr uint64_t kStateOffset = 2;      // number of keys in front of a workgroup
+constexpr uint64_t kStatePoison = 3;      // the offset could not be computed
+constexpr int kIntMin = -2147483647 - 1;
 
 __device__ __forceinline__ uint64_t pack_status(uint64_t state, uint32_t value)
 {
@@ -334,56 +350,74 @@ __device__ __forceinline__ uint64_t peek(const uint64_t* slot)
     return __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Executed by the first wave of a workgroup with ticket > 0.  Returns the sum of the key counts
-// of all workgroups with a smaller ticket.  The wave inspects kLookAhead windows of 64
-// predecessors per round trip to memory (lane l of window u looks at workgroup top - 64u - l)
-// and walks them nearest first; the walk ends at the nearest workgroup that has published a
-// prefix.  The chain of prefixes can only advance one round trip at a time, so the number of
-// predecessors covered per round trip is what bounds how fast workgroups can retire.
-// *failed is set when a predecessor stayed silent for kSpinLimit polls or reported such a failure
-// itself; the wait is bounded so that every wave of the grid exits whatever happens.
-constexpr int kLookAhead = 4;
+// The scanner: one wave.  Reads the workgroups' counts in order, kScanPerLane consecutive ones
+// per lane and trip, and writes the exclusive running sum of every count that is there and has no
+// gap in front of it; then goes on from the first gap.  What counts is how soon after a count an
+// offset follows, i.e. the time of one trip: 128 counts per trip measured fastest on a 3M-Gaussian
+// frame (0.203 ms for the launch against 0.207 with 256, 0.219 with 512 and 0.256 with 1024).
+constexpr int kScanPerLane = 2;
 
-__device__ __forceinline__ uint32_t look_back(const uint64_t* status, int ticket, bool* failed)
+__device__ __forceinline__ void scan_counts(const uint64_t* counts, uint64_t* offsets, int num_blocks,
+                                            int* curr_offset, unsigned spin_limit)
 {
     const int lane = lane_id();
-    uint32_t sum = 0;
+    const uint32_t start = (uint32_t)*curr_offset;      // the caller's starting offset (example.py:69 zeroes it)
+    uint32_t running = start;
     unsigned spins = 0;
-    int top = ticket - 1;
+    int base = 0;
+    bool gave_up = false;
+    while (base < num_blocks) {
+        const int first = base + lane * kScanPerLane;
+        uint64_t w[kScanPerLane];
+#pragma unroll
+        for (int k = 0; k < kScanPerLane; k++) w[k] = first + k < num_blocks ? peek(counts + first + k) : 0;
+        // this lane's entries that exist, and how many of them are there without a gap
+        const int valid = max(0, min(kScanPerLane, num_blocks - first));
+        int ready = 0;
+#pragma unroll
+        for (int k = 0; k < kScanPerLane; k++)
+            if (ready == k && k < valid && (uint32_t)(w[k] >> 32) != 0u) ready = k + 1;
+        const uint64_t gaps = ballot(ready < valid);
+        const int gap_lane = gaps ? __ffsll((long long)gaps) - 1 : kWave;
+        const int take = lane < gap_lane ? valid : (lane == gap_lane ? ready : 0);
+        uint32_t before[kScanPerLane], lane_sum = 0;
+#pragma unroll
+        for (int k = 0; k < kScanPerLane; k++) {
+            before[k] = lane_sum;
+            if (k < take) lane_sum += (uint32_t)w[k];
+        }
+        const uint32_t incl = wave_inclusive_sum(lane_sum);
+        const uint32_t lane_base = running + incl - lane_sum;
+#pragma unroll
+        for (int k = 0; k < kScanPerLane; k++)
+            if (k < take) publish(offsets + first + k, pack_status(kStateOffset, lane_base + before[k]));
+        running += (uint32_t)bcast_i((int)incl, kWave - 1);
+        const int taken = bcast_i((int)wave_inclusive_sum((uint32_t)take), kWave - 1);
+        base += taken;
+        if (taken != 0) spins = 0;
+        else if (++spins > spin_limit) { gave_up = true; break; }
+        else __builtin_amdgcn_s_sleep(1);
+    }
+    if (gave_up) {
+        for (int j = base + lane; j < num_blocks; j += kWave) publish(offsets + j, pack_status(kStatePoison, 0u));
+        if (lane == 0) atomicMin(curr_offset, kIntMin);
+    } else if (lane == 0) {
+        atomicCAS(curr_offset, (int)start, (int)running);
+    }
+}
+
+// Executed by one lane of a workgroup: the number of keys in front of the workgroup, once the
+// scanner has written it.  *failed is set when it did not come within spin_limit polls or is
+// poisoned.
+__device__ __forceinline__ uint32_t wait_for_offset(const uint64_t* slot, unsigned spin_limit, bool* failed)
+{
+    unsigned spins = 0;
     for (;;) {
-        uint64_t w[kLookAhead];
-#pragma unroll
-        for (int u = 0; u < kLookAhead; u++) {
-            const int j = top - u * kWave - lane;
-            w[u] = j >= 0 ? peek(status + j) : 0;
-        }
-#pragma unroll
-        for (int u = 0; u < kLookAhead; u++) {
-            const int j = top - u * kWave - lane;
-            uint64_t word = w[u];
-            uint32_t state;
-            uint64_t closing;        // lanes holding a prefix (or poison) word
-            for (;;) {
-                state = 0;
-                if (j >= 0) state = (uint32_t)(word >> 32) & 3u;
-                const uint64_t pending = ballot(j >= 0 && state == 0);
-                closing = ballot(state >= kStatePrefix);
-                const uint64_t need = closing ? ((closing & (~closing + 1)) << 1) - 1 : ~0ull;
-                if ((pending & need) == 0) break;
-                if (++spins > kSpinLimit) { *failed = true; return sum; }
-                __builtin_amdgcn_s_sleep(2);
-                if (j >= 0) word = peek(status + j);
-            }
-            const uint64_t first = closing & (~closing + 1);
-            const uint64_t take = closing ? (first << 1) - 1 : ~0ull;
-            if (ballot(state == kStatePoison) & first) *failed = true;
-            uint32_t v = (j >= 0 && ((take >> lane) & 1)) ? (uint32_t)word : 0u;
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) v += (uint32_t)__shfl_xor((int)v, o);
-            sum += v;
-            if (closing || top - (u + 1) * kWave < 0) return sum;
-        }
-        top -= kLookAhead * kWave;
+        const uint64_t word = peek(slot);
+        const uint32_t state = (uint32_t)(word >> 32) & 3u;
+        if (state == kStateOffset) return (uint32_t)word;
+        if (state == kStatePoison || ++spins > spin_limit) { *failed = true; return 0u; }
+        __builtin_amdgcn_s_sleep(2);
     }
 }
 
@@ -401,9 +435,10 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     uint32_t* __restrict__ values,
     int* __restrict__ curr_offset,
     int64_t capacity,            // <= 0: unchecked
-    uint64_t* __restrict__ scan_words,     // control word, then two status arrays of status_capacity words
+    uint64_t* __restrict__ scan_words,     // control word, then two generations of (counts, offsets), status_capacity words each
     int status_capacity,
-    int num_blocks)
+    int num_blocks,                        // workgroups that hold Gaussians; the grid has one more, the scanner's
+    unsigned spin_limit)
 {
     __shared__ uint32_t s_wave_total[kWavesPerBlock];
     __shared__ uint32_t s_block_base;
@@ -427,19 +462,28 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     if (tid == 0) s_nhuge = 0;
     __syncthreads();
 
-    // Workgroups are numbered by their index: the hardware dispatches them in index order, so
-    // every workgroup with a smaller index is already running or finished when this one waits
-    // for it (and the wait is bounded in any case).
-    const int ticket = (int)blockIdx.x;
-    const int idx = ticket * kBlock + tid;
-    // this launch's status array; the other one is cleared for the launch that follows
+    // this launch's generation of the scan words; the other one is cleared for the launch that follows
     const uint32_t which = (uint32_t)peek(scan_words) & 1u;
-    uint64_t* const status = scan_words + kControlWords + (size_t)which * status_capacity;
+    uint64_t* const counts = scan_words + kControlWords + (size_t)which * 2 * status_capacity;
+    uint64_t* const offsets = counts + status_capacity;
     {
-        uint64_t* const other = scan_words + kControlWords + (size_t)(which ^ 1u) * status_capacity;
-        for (long long w = ticket + (long long)tid * num_blocks; w < status_capacity; w += (long long)kBlock * num_blocks)
-            other[w] = 0;
+        uint64_t* const other = scan_words + kControlWords + (size_t)(which ^ 1u) * 2 * status_capacity;
+        const long long words = 2LL * status_capacity, threads = (long long)kBlock * (num_blocks + 1);
+        for (long long w = (long long)blockIdx.x * kBlock + tid; w < words; w += threads) other[w] = 0;
     }
+    // Workgroup 0 is the scanner.  The hardware dispatches workgroups in index order, so it runs
+    // from the start, and every workgroup whose count it waits for is running or finished when a
+    // later one waits for its offset (and every wait is bounded in any case).
+    if (blockIdx.x == 0) {
+        if (wave == 0) {
+            scan_counts(counts, offsets, num_blocks, curr_offset, spin_limit);
+            // every workgroup has read the control word by now: hand the other generation to the next launch
+            if (lane == 0) publish(scan_words, (uint64_t)(which ^ 1u));
+        }
+        return;
+    }
+    const int ticket = (int)blockIdx.x - 1;
+    const int idx = ticket * kBlock + tid;
     // tile coordinates travel in 12 bits each and tile indices in 26 when candidates are laid flat
     const bool pack_ok = cam.gx <= 4096 && cam.gy <= 4096 && (long long)cam.gx * cam.gy <= (1 << 26);
 
@@ -755,7 +799,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         }
     }
 
-    // ---- slots: wave scan, block scan, chained scan over workgroups ----
+    // ---- slots: wave scan, block scan, scan over workgroups ----
     uint32_t incl = wave_inclusive_sum(count);
     const uint32_t wave_total = (uint32_t)bcast_i((int)incl, kWave - 1);
     if (lane == 0) s_wave_total[wave] = wave_total;
@@ -769,9 +813,9 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         block_total += t;
     }
 
-    // The workgroup's count is published right away; the wait for the counts of earlier
-    // workgroups comes after the colour work below, when they have long been published.
-    if (tid == 0 && ticket != 0) publish(status + ticket, pack_status(kStateAggregate, block_total));
+    // The workgroup's count is published right away; its offset is picked up after the colour
+    // work below, when the scanner has long written it.
+    if (tid == 0) publish(counts + ticket, pack_status(kStateCount, block_total));
 
     // ---- attributes of Gaussians that emit a key (preprocess.cu:411-417) ----
     if (count > 0) {
@@ -784,21 +828,10 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         reinterpret_cast<float4*>(rgb_depth)[idx] = make_float4(rgb[0], rgb[1], rgb[2], depth);
     }
 
-    if (wave == 0) {
-        bool timed_out = false;
-        uint32_t excl;
-        if (ticket == 0) excl = (uint32_t)*curr_offset;     // the caller's starting offset (example.py:69 zeroes it)
-        else excl = look_back(status, ticket, &timed_out);
-        if (lane == 0) {
-            publish(status + ticket, pack_status(timed_out ? kStatePoison : kStatePrefix, excl + block_total));
-            s_block_base = excl;
-            // only the last workgroup writes the counter (a poisoned chain yields a negative count)
-            // and hands the other status array to the next launch
-            if (ticket == num_blocks - 1) {
-                *curr_offset = timed_out ? -2147483647 - 1 : (int)(excl + block_total);
-                publish(scan_words, (uint64_t)(which ^ 1u));
-            }
-        }
+    if (tid == 0) {
+        bool failed = false;
+        s_block_base = wait_for_offset(offsets + ticket, spin_limit, &failed);
+        if (failed) atomicMin(curr_offset, kIntMin);
     }
     __syncthreads();
     const uint32_t my_slot = s_block_base + wave_base + (incl - count);
@@ -882,16 +915,17 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
 
 }
 
-// ---- per-device scratch for the chained scan ------------------------------------------------------
+// ---- per-device scan words ------------------------------------------------------------------------
 
 struct Scratch {
-    uint64_t* words = nullptr;      // control word (+ padding), then two status arrays
-    size_t capacity = 0;            // workgroups each status array holds
+    uint64_t* words = nullptr;      // control word (+ padding), then two generations of (counts, offsets)
+    size_t capacity = 0;            // workgroups each of the four arrays holds
 };
 
 constexpr int kMaxDevices = 64;
 Scratch g_scratch[kMaxDevices];
 std::mutex g_mutex;
+std::atomic<unsigned> g_spin_limit{kSpinLimit};
 
 int acquire_scratch(int device, int num_blocks, hipStream_t stream, Scratch** out)
 {
@@ -904,7 +938,7 @@ int acquire_scratch(int device, int num_blocks, hipStream_t stream, Scratch** ou
         s.capacity = 0;
         size_t cap = 4096;
         while (cap < (size_t)num_blocks) cap <<= 1;
-        const size_t bytes = (kControlWords + 2 * cap) * sizeof(uint64_t);
+        const size_t bytes = (kControlWords + 4 * cap) * sizeof(uint64_t);
         if (hipMalloc((void**)&s.words, bytes) != hipSuccess) {
             (void)hipGetLastError();
             return fail(FGS_E_NOMEM, "cannot allocate %zu bytes of scan status", bytes);
@@ -969,13 +1003,13 @@ namespace {
 
 // ---- scan status held in the library's own image, for callers that cannot allocate ----------------
 //
-// The same two status arrays as the allocated scratch, as a file-scope device array: one copy per
+// The same scan words as the allocated ones, as a file-scope device array: one copy per
 // GPU that loads the library, zero when the code object is loaded, kept until the process ends.
 // In host code the array's name is only a handle; the device address comes from
 // hipGetSymbolAddress, once per device with that device current.
-constexpr int kStaticBlocks = 1 << 16;                        // workgroups one status array holds
+constexpr int kStaticBlocks = 1 << 16;                        // workgroups each of the four arrays holds
 constexpr int kStaticMaxP = kStaticBlocks * kBlock;           // 16 777 216 Gaussians
-static __device__ __align__(256) uint64_t scratch[kControlWords + 2 * kStaticBlocks];
+static __device__ __align__(256) uint64_t scratch[kControlWords + 4 * kStaticBlocks];
 uint64_t* g_static_words[kMaxDevices];                        // device address of `scratch`, per device
 
 int static_scratch(int device, uint64_t** out)
@@ -1049,15 +1083,20 @@ int preprocess_impl(bool allocate, const char* who, int P,
         status_capacity = kStaticBlocks;
     }
 
-    hipLaunchKernelGGL(preprocess_kernel, dim3(num_blocks), dim3(kBlock), 0, st,
+    hipLaunchKernelGGL(preprocess_kernel, dim3(num_blocks + 1), dim3(kBlock), 0, st,
                        P, positions, shs, opacities, cov3Ds, cam, points_xy, rgb_depth, conic_opacity,
                        gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset, key_capacity,
-                       words, status_capacity, num_blocks);
+                       words, status_capacity, num_blocks, g_spin_limit.load());
     return check_hip(hipGetLastError(), "preprocess_kernel launch");
 }
 
 } // namespace
 } // namespace fgs
+
+extern "C" unsigned fgs_set_scan_spin_limit(unsigned polls)
+{
+    return fgs::g_spin_limit.exchange(polls);
+}
 
 extern "C" int fgs_preprocess(int P,
                               const float* positions, const float* shs, const float* opacities, const float* cov3Ds,

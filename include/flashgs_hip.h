@@ -50,8 +50,8 @@ extern "C" {
  * scan over workgroups (allocated on first use, grown when a larger P arrives - the only times
  * the call synchronises); calls on one device must not overlap in time.  Nothing on the host
  * changes from launch to launch, so once the scratch is large enough a launch can be captured in
- * a HIP graph and replayed.  If the scan ever times out waiting for a workgroup, *curr_offset is
- * set to INT_MIN.
+ * a HIP graph and replayed.  Every wait inside the launch is bounded (fgs_set_scan_spin_limit);
+ * if one ever gives up, *curr_offset ends negative and the keys are not to be used.
  */
 int fgs_preprocess(int P,
                    const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
@@ -65,7 +65,7 @@ int fgs_preprocess(int P,
 /*
  * No counterpart in the reference.  fgs_preprocess for callers that cannot allocate device
  * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
- * same arguments, same kernel, same results, but the scan status lives in a 1 MiB array inside
+ * same arguments, same kernel, same results, but the scan status lives in a 2 MiB array inside
  * the library's device image (one copy per GPU, held until the process ends) instead of a
  * buffer from hipMalloc, so the call allocates and frees nothing and never synchronises.
  * P is limited to 16 777 216 Gaussians; a larger P returns FGS_E_INVALID.  Every call on one GPU
@@ -157,6 +157,16 @@ int fgs_blend(int block_x, int block_y, int width, int height,
 void fgs_camera_matrices(const float cam_position[3], const float cam_rotation[9],
                          int width, int height, float focal_x, float focal_y, float zFar, float zNear,
                          float view[16], float proj[16]);
+
+/*
+ * No counterpart in the reference.  Number of polls after which a wait inside the preprocess
+ * launch (the scanner for a workgroup's key count, a workgroup for its key offset) gives up and
+ * the launch reports a negative pair count; applies to launches made after the call, returns the
+ * previous value.  The default, 1 << 22, is seconds of waiting and is never reached by a healthy
+ * launch.  A diagnostic knob: 0 makes every wait that is not satisfied at its first poll give up,
+ * which is how the give-up path is tested without hanging anything.
+ */
+unsigned fgs_set_scan_spin_limit(unsigned polls);
 
 /* Message of the last failing call on this thread ("" if none). */
 const char* fgs_last_error(void);

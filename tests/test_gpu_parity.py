@@ -209,6 +209,35 @@ def test_start_offset_and_capacity_guard(oracle):
     assert np.all(gp.u64(keys)[cap:] == 0) and np.all(values.cpu().numpy()[cap:] == -1)   # nothing past the capacity
 
 
+def test_scan_waits_that_give_up_report_a_negative_count(oracle):
+    """With the spin limit at 0 every wait of the preprocess launch that is not satisfied at its
+    first poll gives up: the kernel still runs to its end (no wave is left waiting), the pair
+    count comes back negative - which the sort refuses - and the next launch with the normal
+    limit is correct again, both entry points."""
+    import gpu_pipeline as gp
+    from flashgs_amd import cabi
+    sc = scenes.config0(n=120_000)
+    cam = sc.cameras[0]
+    sd = gp.SceneOnDevice(sc)
+    good = gp.preprocess(sd, cam, 1 << 20)
+    K = good["num_rendered"]
+    assert K > 100_000
+    for static in (False, True):
+        previous = cabi.set_scan_spin_limit(0)
+        try:
+            bad = gp.preprocess(sd, cam, 1 << 20, static=static)
+        finally:
+            assert cabi.set_scan_spin_limit(previous) == 0
+        assert previous == 1 << 22
+        assert bad["num_rendered"] < 0
+        with pytest.raises(RuntimeError, match="negative"):
+            gp.sort(bad["num_rendered"], cam.width, cam.height, bad["keys"], bad["values"])
+        again = gp.preprocess(sd, cam, 1 << 20, static=static)
+        assert again["num_rendered"] == K
+        assert np.array_equal(gp.u64(again["keys"])[:K], gp.u64(good["keys"])[:K])
+        assert np.array_equal(gp.u32(again["values"])[:K], gp.u32(good["values"])[:K])
+
+
 def test_preprocess_replayed_from_a_captured_graph():
     """fgs_preprocess keeps no per-launch state on the host, so a captured launch can be replayed:
     every replay (with eager launches of other sizes in between) gives the eager result."""
