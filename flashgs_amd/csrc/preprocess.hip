@@ -23,7 +23,9 @@
 #include "fgs_internal.h"
 
 #include <atomic>
+#include <map>
 #include <mutex>
+#include <utility>
 
 namespace fgs {
 namespace {
@@ -915,7 +917,12 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
 
 }
 
-// ---- per-device scan words ------------------------------------------------------------------------
+// ---- scan words, one set per (device, stream) -------------------------------------------------------
+//
+// Launches on one stream follow each other, so they can share one set of scan words; launches on
+// different streams of a device may overlap in time and get a set each.  A set is allocated on
+// the first call on its stream and grown when a larger P arrives (the only times a call
+// synchronises), and lives until the process ends.
 
 struct Scratch {
     uint64_t* words = nullptr;      // control word (+ padding), then two generations of (counts, offsets)
@@ -923,14 +930,20 @@ struct Scratch {
 };
 
 constexpr int kMaxDevices = 64;
-Scratch g_scratch[kMaxDevices];
+std::map<std::pair<int, hipStream_t>, Scratch> g_scratch;
 std::mutex g_mutex;
 std::atomic<unsigned> g_spin_limit{kSpinLimit};
 
+// *out stays null when the stream is being captured and has no (large enough) set yet: nothing
+// can be allocated then, and the caller falls back to the words inside the library's image.
 int acquire_scratch(int device, int num_blocks, hipStream_t stream, Scratch** out)
 {
-    Scratch& s = g_scratch[device];
+    *out = nullptr;
+    Scratch& s = g_scratch[std::make_pair(device, stream)];
     if (s.capacity < (size_t)num_blocks) {
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        if (stream) FGS_HIP_TRY(hipStreamIsCapturing(stream, &capture));
+        if (capture != hipStreamCaptureStatusNone) return FGS_OK;
         // the stream may still be reading the old arrays: drain it before the swap
         FGS_HIP_TRY(hipStreamSynchronize(stream));
         if (s.words) FGS_HIP_TRY(hipFree(s.words));
@@ -1071,12 +1084,17 @@ int preprocess_impl(bool allocate, const char* who, int P,
     std::lock_guard<std::mutex> lock(g_mutex);
     uint64_t* words = nullptr;
     int status_capacity = 0;
+    Scratch* own = nullptr;
     if (allocate) {
-        Scratch* s = nullptr;
-        int rc = acquire_scratch(device, num_blocks, st, &s);
+        int rc = acquire_scratch(device, num_blocks, st, &own);
         if (rc != FGS_OK) return rc;
-        words = s->words;
-        status_capacity = (int)s->capacity;
+        if (!own && P > kStaticMaxP)
+            return fail(FGS_E_INVALID, "%s: the stream is being captured and no call with P >= %d has run on it "
+                                       "before, so nothing can be allocated; run one such call first", who, P);
+    }
+    if (own) {
+        words = own->words;
+        status_capacity = (int)own->capacity;
     } else {
         int rc = static_scratch(device, &words);
         if (rc != FGS_OK) return rc;

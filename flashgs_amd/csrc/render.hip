@@ -13,6 +13,10 @@
 // workgroup is a single wave, so no workgroup barrier is needed anywhere.
 #include "fgs_internal.h"
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 namespace fgs {
 namespace {
 
@@ -31,9 +35,42 @@ __global__ __launch_bounds__(256) void fill_i32_kernel(int* p, size_t n, int v)
 // workgroup then has to push its ranges out of its XCD's L2 before it counts itself done.)
 constexpr int kOrderCap = 8192;            // tiles
 constexpr int kOrderBins = 128;            // everything from 2032 entries up shares the first bin
+// The ranking is written by one launch and read by the next, so it needs memory of its own: one
+// table per (device, stream), allocated on the first such blend on that stream (blends on one
+// stream follow each other; blends on different streams may overlap and get a table each).  A
+// stream that is being captured and has no table yet cannot allocate one and uses this
+// per-device table instead, which captured blends on one device then share.
 __device__ uint32_t g_tile_order[kOrderCap];
+std::map<std::pair<int, hipStream_t>, uint32_t*> g_order_tables;
+std::mutex g_order_mutex;
 
-__global__ __launch_bounds__(1024) void tile_order_kernel(const int2* __restrict__ ranges, int num_tiles)
+int tile_order_table(hipStream_t stream, uint32_t** out)
+{
+    int device = 0;
+    FGS_HIP_TRY(hipGetDevice(&device));
+    std::lock_guard<std::mutex> lock(g_order_mutex);
+    uint32_t*& table = g_order_tables[std::make_pair(device, stream)];
+    if (!table) {
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        if (stream) FGS_HIP_TRY(hipStreamIsCapturing(stream, &capture));
+        if (capture != hipStreamCaptureStatusNone) {
+            void* shared = nullptr;
+            FGS_HIP_TRY(hipGetSymbolAddress(&shared, HIP_SYMBOL(g_tile_order)));
+            *out = (uint32_t*)shared;
+            return FGS_OK;
+        }
+        if (hipMalloc((void**)&table, kOrderCap * sizeof(uint32_t)) != hipSuccess) {
+            (void)hipGetLastError();
+            table = nullptr;
+            return fail(FGS_E_NOMEM, "cannot allocate the table of tile ranks");
+        }
+    }
+    *out = table;
+    return FGS_OK;
+}
+
+__global__ __launch_bounds__(1024) void tile_order_kernel(const int2* __restrict__ ranges, int num_tiles,
+                                                          uint32_t* __restrict__ tile_order)
 {
     constexpr int kPerThread = kOrderCap / 1024;
     __shared__ uint32_t s_count[kOrderBins];
@@ -69,7 +106,7 @@ __global__ __launch_bounds__(1024) void tile_order_kernel(const int2* __restrict
 #pragma unroll
     for (int k = 0; k < kPerThread; k++) {
         const int t = tid + k * 1024;
-        if (t < num_tiles) g_tile_order[s_count[bin[k]] + slot[k]] = (uint32_t)t;
+        if (t < num_tiles) tile_order[s_count[bin[k]] + slot[k]] = (uint32_t)t;
     }
 }
 
@@ -472,7 +509,7 @@ constexpr int kOwnShare = 256;
 constexpr int kMinRest = 512;               // a shorter rest is not worth two barriers: the owner walks it
 constexpr int kSharedWaves = 4;
 
-__global__ __launch_bounds__(kSharedWaves * kWave) void blend_kernel_shared(FGS_BLEND_PARAMS)
+__global__ __launch_bounds__(kSharedWaves * kWave) void blend_kernel_shared(FGS_BLEND_PARAMS, const uint32_t* __restrict__ tile_order)
 {
     using Role = LaneRole<1, 1>;
     __shared__ __align__(16) float s_rec[kSharedWaves][kBatch * Role::kRec];
@@ -486,7 +523,7 @@ __global__ __launch_bounds__(kSharedWaves * kWave) void blend_kernel_shared(FGS_
     const bool active = rank < tiles_x * tiles_y;
     int tile_x = 0, tile_y = 0;
     if (active) {
-        const int tile = (int)g_tile_order[rank];
+        const int tile = (int)tile_order[rank];
         tile_x = tile % tiles_x;
         tile_y = tile / tiles_x;
     }
@@ -664,11 +701,14 @@ int blend_impl(int block_x, int block_y, int width, int height,
     } while (0)
     if (shape.shared) {
         const int num_tiles = tiles_x * tiles_y;
-        hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, st, (const int2*)ranges, num_tiles);
+        uint32_t* tile_order = nullptr;
+        rc = tile_order_table(st, &tile_order);
+        if (rc != FGS_OK) return rc;
+        hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, st, (const int2*)ranges, num_tiles, tile_order);
         hipLaunchKernelGGL(blend_kernel_shared, dim3((unsigned)((num_tiles + kSharedWaves - 1) / kSharedWaves)), dim3(kSharedWaves * kWave), 0, st,
                            (const int2*)ranges, values_sorted, width, height, tiles_x, tiles_y,
                            (const float2*)points_xy, (const float4*)rgb_depth, (const float4*)conic_opacity,
-                           bg[0], bg[1], bg[2], out_u8, out_f32);
+                           bg[0], bg[1], bg[2], out_u8, out_f32, (const uint32_t*)tile_order);
     } else if (sx == 1 && sy == 1) FGS_LAUNCH_BLEND(1, 1);
     else if (sx == 2 && sy == 1) FGS_LAUNCH_BLEND(2, 1);
     else FGS_LAUNCH_BLEND(2, 2);

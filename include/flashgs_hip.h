@@ -46,12 +46,15 @@ extern "C" {
  * counts them, so the caller's check of example.py:79-82 keeps working); pass 0 to write
  * unchecked like the reference (preprocess.cu:330,395).
  *
- * The call is asynchronous on `stream`.  The library keeps a small per-device scratch for the
- * scan over workgroups (allocated on first use, grown when a larger P arrives - the only times
- * the call synchronises); calls on one device must not overlap in time.  Nothing on the host
- * changes from launch to launch, so once the scratch is large enough a launch can be captured in
- * a HIP graph and replayed.  Every wait inside the launch is bounded (fgs_set_scan_spin_limit);
- * if one ever gives up, *curr_offset ends negative and the keys are not to be used.
+ * The call is asynchronous on `stream`.  The library keeps a small scratch for the scan over
+ * workgroups per (device, stream), allocated on the first call on that stream and grown when a
+ * larger P arrives - the only times the call synchronises - so calls on different streams of one
+ * device may overlap in time.  Nothing on the host changes from launch to launch, so a launch can
+ * be captured in a HIP graph and replayed; a stream that is being captured and has no (large
+ * enough) scratch yet cannot allocate one and uses the built-in scan status of
+ * fgs_preprocess_static, with its limits.  Every wait inside the launch is bounded
+ * (fgs_set_scan_spin_limit); if one ever gives up, *curr_offset ends negative and the keys are
+ * not to be used.
  */
 int fgs_preprocess(int P,
                    const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
@@ -106,11 +109,12 @@ size_t fgs_get_sort_buffer_size(int num_rendered);
  * sorted keys, blend front to back and write out_color u8[H,W,3].  `ranges` int32[tiles,2] is
  * scratch that holds the tile ranges afterwards.  bg_color is a host array of 3 floats.
  * A frame of at most 8192 16x16 tiles first ranks its tiles by list length into a table the
- * library keeps per device (4 bytes per tile), and the rest of a list of more than 768 entries
- * is blended in four runs that each stop on their own transmittance: the colour can differ from
- * the pair-by-pair walk of render.cu:315-408 by what lies behind T < 1e-4, i.e. by less than
- * 1e-4 of a colour.  Because of the table, blends on one device must not overlap in time (calls
- * on one stream, or otherwise ordered, never do).
+ * library keeps per (device, stream) (32 KB, allocated on the first such call on that stream),
+ * and the rest of a list of more than 768 entries is blended in four runs that each stop on
+ * their own transmittance: the colour can differ from the pair-by-pair walk of
+ * render.cu:315-408 by what lies behind T < 1e-4, i.e. by less than 1e-4 of a colour.  Calls on
+ * different streams may overlap in time; a stream that is being captured and has no table yet
+ * uses one table per device instead, so replays of such graphs on one device must not overlap.
  */
 int fgs_render_16x16(int num_rendered, int width, int height,
                      const float* points_xy, const float* rgb_depth, const float* conic_opacity,

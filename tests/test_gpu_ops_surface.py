@@ -150,3 +150,46 @@ def test_render_scene_from_ply_and_cameras_json(oracle, tmp_path, capsys):
         d = np.abs(img.astype(np.int16) - u8.astype(np.int16))
         assert d.max() <= 1 and (d > 0).mean() < 0.01
         assert img.max() > 100          # not an empty frame
+
+
+def test_two_rasterizers_on_two_streams_overlapping(oracle):
+    """Two renderers with their own buffers on two streams of one device, frames enqueued back to
+    back without any ordering between the streams: the library keeps its scratch per stream, so
+    both produce exactly what each produces alone (and what the oracle produces)."""
+    sc_a = scenes.config0(n=60_000)
+    sc_b = scenes.make(1, n=150_000)
+    dev = torch.device("cuda:0")
+    jobs = []
+    for sc in (sc_a, sc_b):
+        scene = Scene(dev).from_arrays(sc.position, sc.shs, sc.opacity, sc.cov3d)
+        cam = Camera.from_synthetic(sc.cameras[0])
+        rast = Rasterizer(scene, 1 << 21, 1 << 14)
+        jobs.append((sc, scene, cam, rast, torch.cuda.Stream()))
+    bg = torch.tensor([0.1, 0.3, 0.5])
+    alone = []
+    for sc, scene, cam, rast, _ in jobs:
+        alone.append(rast.forward(scene, cam, bg).clone())
+        assert rast.num_rendered > 50_000
+    torch.cuda.synchronize()
+    # both frames are small enough to rank their tiles (the table the blend keeps per stream)
+    outs = [[], []]
+    for rep in range(6):
+        for k, (sc, scene, cam, rast, stream) in enumerate(jobs):
+            with torch.cuda.stream(stream):
+                outs[k].append(rast.forward(scene, cam, bg).clone())
+    torch.cuda.synchronize()
+    for k in range(2):
+        for img in outs[k]:
+            assert torch.equal(img, alone[k])
+    # and the image is the oracle's
+    sc, scene, cam, rast, _ = jobs[0]
+    c0 = sc.cameras[0]
+    pre = oracle.preprocess(sc.position, sc.shs, sc.opacity, sc.cov3d, c0.width, c0.height, 16, 16,
+                            c0.position, c0.rotation, c0.focal_x, c0.focal_y, c0.zFar, c0.zNear, 1 << 21)
+    K = pre["num_rendered"]
+    ks, vs = oracle.sort(K, c0.width, c0.height, 16, 16, pre["keys"], pre["values"])
+    rg = oracle.ranges(K, ks, ((c0.width + 15) // 16) * ((c0.height + 15) // 16))
+    u8, _, _ = oracle.render(c0.width, c0.height, 16, 16, pre["points_xy"], pre["rgb_depth"], pre["conic_opacity"], vs, rg,
+                             bg.numpy(), want_f32=False)
+    d = np.abs(alone[0].cpu().numpy().astype(np.int16) - u8.astype(np.int16))
+    assert d.max() <= 1 and (d > 0).mean() < 0.01
