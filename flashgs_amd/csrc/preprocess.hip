@@ -52,8 +52,19 @@ struct Camera {
 
 // ---- scalar numerics ---------------------------------------------------------------------------
 
-__device__ __forceinline__ float min_f(float a, float b) { return a < b ? a : b; }
-__device__ __forceinline__ float max_f(float a, float b) { return a > b ? a : b; }
+// min / max of preprocess.cu:116-117 and max.f32 of :36-41: a NaN operand yields the other one
+__device__ __forceinline__ float min_f(float a, float b)
+{
+    if (!(a == a)) return b;
+    if (!(b == b)) return a;
+    return a < b ? a : b;
+}
+__device__ __forceinline__ float max_f(float a, float b)
+{
+    if (!(a == a)) return b;
+    if (!(b == b)) return a;
+    return a > b ? a : b;
+}
 
 // Saturating float -> int: NaN -> 0, out-of-range clamps (the behaviour preprocess.cu:93-98 and
 // :309-310 get from the device conversion instruction).
@@ -819,8 +830,9 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     // work below, when the scanner has long written it.
     if (tid == 0) publish(counts + ticket, pack_status(kStateCount, block_total));
 
-    // ---- attributes of Gaussians that emit a key (preprocess.cu:411-417) ----
-    if (count > 0) {
+    // ---- attributes of Gaussians that emit a key, and of every Gaussian whose rectangle is a
+    // single tile, hit or not (preprocess.cu:317, 411-417: vertex_valid starts as single_tile) ----
+    if (count > 0 || area == 1) {
         constexpr float log2e = 1.4426950216293334961f;
         reinterpret_cast<float2*>(points_xy)[idx] = make_float2(cx, cy);
         reinterpret_cast<float4*>(conic_opacity)[idx] =

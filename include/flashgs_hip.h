@@ -36,7 +36,8 @@ extern "C" {
  *
  * positions f32[P,3], shs f32[P,48], opacities f32[P], cov3Ds f32[P,6] are device inputs;
  * points_xy f32[P,2], rgb_depth f32[P,4], conic_opacity f32[P,4] are device outputs whose rows
- * are written only for Gaussians that emit at least one key; keys/values receive the
+ * are written only for Gaussians that emit at least one key or whose candidate rectangle is a
+ * single tile (preprocess.cu:317,411-417); all other rows keep what they held; keys/values receive the
  * (tile << 32 | depth bits, Gaussian index) pairs starting at *curr_offset, in ascending
  * Gaussian index then row-major tile order; *curr_offset (device int, zeroed by the caller as
  * in example.py:69) ends at the total number of pairs.

@@ -57,8 +57,19 @@ inline int f2i_sat(float f)
     return (int)f;
 }
 
-inline float fminf_(float a, float b) { return a < b ? a : b; }
-inline float fmaxf_(float a, float b) { return a > b ? a : b; }
+/* min / max of preprocess.cu:116-117 and max.f32 of :36-41: a NaN operand yields the other one. */
+inline float fminf_(float a, float b)
+{
+    if (!(a == a)) return b;
+    if (!(b == b)) return a;
+    return a < b ? a : b;
+}
+inline float fmaxf_(float a, float b)
+{
+    if (!(a == a)) return b;
+    if (!(b == b)) return a;
+    return a > b ? a : b;
+}
 inline int imin(int a, int b) { return a < b ? a : b; }
 inline int imax(int a, int b) { return a > b ? a : b; }
 
@@ -496,7 +507,10 @@ int fgs_oracle_preprocess(int P, const float* positions, const float* shs,
                     any = true;
                 }
             }
-            if (any) {   /* preprocess.cu:411-417 */
+            /* preprocess.cu:317,411-417: a rectangle of one tile gets its record whether or not
+             * the tile passed the test (vertex_valid starts as single_tile) */
+            const bool single_tile = (g.rmax[0] - g.rmin[0]) * (g.rmax[1] - g.rmin[1]) == 1;
+            if (any || single_tile) {
                 nvis[t]++;
                 points_xy[2 * i + 0] = g.point_xy[0];
                 points_xy[2 * i + 1] = g.point_xy[1];

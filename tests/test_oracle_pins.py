@@ -301,16 +301,49 @@ def test_key_list_invariants_and_stale_rows(oracle):
     same = np.diff(vals.astype(np.int64)) == 0
     assert np.all(np.diff((keys >> 32).astype(np.int64))[same] > 0)    # row-major tiles inside one Gaussian
     assert np.array_equal(depth, r["rgb_depth"][vals, 3])
-    visible = np.zeros(n, bool)
-    visible[vals] = True
-    assert visible.sum() == r["counts"]["visible"]
+    emitting = np.zeros(n, bool)
+    emitting[vals] = True
+    # rows are written for the Gaussians that emit, plus the few whose one-tile rectangle failed
+    # the test (test_one_tile_rectangle_gets_its_record_without_a_key); every other row is stale
+    written = r["rgb_depth"][:, 3] != sentinel
+    assert written.sum() == r["counts"]["visible"]
+    assert np.all(written[emitting]) and (written & ~emitting).sum() <= 0.01 * emitting.sum()
     for name in ("points_xy", "rgb_depth", "conic_opacity"):
-        assert np.all(r[name][~visible] == sentinel)
-        assert not np.any(r[name][visible][:, -1] == sentinel)
+        assert np.all(r[name][~written] == sentinel)
+        assert not np.any(r[name][written][:, -1] == sentinel)
     # single-threaded and multi-threaded runs give the same list
     r1 = oracle.preprocess(sc.position, sc.shs, sc.opacity, sc.cov3d, cam.width, cam.height, 16, 16, cam.position,
                            cam.rotation, cam.focal_x, cam.focal_y, cam.zFar, cam.zNear, 1 << 18, threads=1)
     assert np.array_equal(r1["keys"][:K], keys) and np.array_equal(r1["values"][:K], vals)
+
+
+def test_one_tile_rectangle_gets_its_record_without_a_key(oracle):
+    """preprocess.cu:317,411-417: vertex_valid starts as single_tile, so a Gaussian whose candidate
+    rectangle is one tile has its attribute rows written even when that tile fails the ellipse
+    test.  A small splat 12 pixels left of the image: the rectangle is clamped to tile (0, 6), which
+    the ellipse (about 6 pixels at the opacity threshold) does not reach."""
+    W, H, f, z = 1280, 720, 800.0, 10.0
+    p = np.array([[(-12.0 - (W - 1) / 2) * z / f, (104.0 - (H - 1) / 2) * z / f, z]], np.float32)
+    s2 = (math.sqrt(3.4) * z / f) ** 2
+    cov3d = np.array([[s2, 0, 0, s2, 0, s2]], np.float32)
+    sentinel = np.float32(-7.5)
+    r = oracle.preprocess(p, np.zeros((1, 48), np.float32), np.array([0.6], np.float32), cov3d, W, H, 16, 16,
+                          (0, 0, 0), np.eye(3), f, f, 100.0, 0.01, 16, threads=1,
+                          points_xy=np.full((1, 2), sentinel), rgb_depth=np.full((1, 4), sentinel),
+                          conic_opacity=np.full((1, 4), sentinel))
+    assert r["counts"]["candidates"] == 1 and r["num_rendered"] == 0
+    assert r["counts"]["visible"] == 1
+    np.testing.assert_allclose(r["points_xy"][0], [-12.0, 104.0], atol=1e-3)
+    assert r["rgb_depth"][0, 3] == np.float32(z) and r["conic_opacity"][0, 3] == np.float32(oracle.log2f(np.float32(0.6)))
+    # two tiles high instead (centre on a tile border): no key, and now no record either
+    p2 = p.copy()
+    p2[0, 1] = (96.0 - (H - 1) / 2) * z / f
+    r = oracle.preprocess(p2, np.zeros((1, 48), np.float32), np.array([0.6], np.float32), cov3d, W, H, 16, 16,
+                          (0, 0, 0), np.eye(3), f, f, 100.0, 0.01, 16, threads=1,
+                          points_xy=np.full((1, 2), sentinel), rgb_depth=np.full((1, 4), sentinel),
+                          conic_opacity=np.full((1, 4), sentinel))
+    assert r["counts"]["candidates"] == 2 and r["num_rendered"] == 0 and r["counts"]["visible"] == 0
+    assert np.all(r["rgb_depth"] == sentinel) and np.all(r["points_xy"] == sentinel)
 
 
 def test_cull_rules(oracle):
@@ -471,6 +504,54 @@ def test_blend_one_gaussian_closed_form(oracle):
     np.testing.assert_allclose(f32, want, atol=2e-6)
     assert np.array_equal(u8, np.minimum(np.maximum(f32 * np.float32(255.0), 0), 255).astype(np.uint8))
     assert walked == 12
+
+
+def test_rotated_gaussian_image_closed_form(oracle):
+    """One anisotropic, rotated Gaussian through preprocess -> sort -> ranges -> render: inside the
+    emitted tiles the image is op * exp(-1/2 d^T S^-1 d) * rgb + (1 - alpha) * bg with S the EWA
+    covariance J W Sigma W^T J^T + 0.3 I inverted in float64.  The off-diagonal term of S^-1 enters
+    the blend as conic.y * dx * dy: a wrong sign or a swapped axis there mirrors the ellipse."""
+    W, H, f = 256, 192, 400.0
+    rng = np.random.default_rng(5)
+    bg = np.array([0.1, 0.2, 0.7])
+    for trial in range(4):
+        p = np.array([rng.uniform(-1, 1), rng.uniform(-0.6, 0.6), rng.uniform(6, 9)])
+        th = rng.uniform(0.3, 1.2) * (1 if trial % 2 else -1)              # rotation about the view axis: both signs
+        tilt = rng.uniform(-0.4, 0.4)                                       # and a little out of the image plane
+        Rz = np.array([[math.cos(th), -math.sin(th), 0], [math.sin(th), math.cos(th), 0], [0, 0, 1]])
+        Rx = np.array([[1, 0, 0], [0, math.cos(tilt), -math.sin(tilt)], [0, math.sin(tilt), math.cos(tilt)]])
+        R = Rz @ Rx
+        S3 = R @ np.diag([0.35, 0.06, 0.12]) ** 2 @ R.T
+        cov3d = np.array([[S3[0, 0], S3[0, 1], S3[0, 2], S3[1, 1], S3[1, 2], S3[2, 2]]], np.float32)
+        op = 0.85
+        sh = np.zeros((1, 48), np.float32)
+        sh[0, :3] = (np.array([0.9, 0.5, 0.2]) - 0.5) / 0.28209479177387814      # degree 0 only: colour = 0.5 + C0 * dc
+        pre = oracle.preprocess(p[None].astype(np.float32), sh, np.array([op], np.float32), cov3d, W, H, 16, 16,
+                                (0, 0, 0), np.eye(3), f, f, 100.0, 0.01, 4096, threads=1)
+        K = pre["num_rendered"]
+        assert K >= 4
+        ks, vs = oracle.sort(K, W, H, 16, 16, pre["keys"], pre["values"])
+        gx, gy = W // 16, H // 16
+        rg = oracle.ranges(K, ks, gx * gy)
+        _, img, _ = oracle.render(W, H, 16, 16, pre["points_xy"], pre["rgb_depth"], pre["conic_opacity"], vs, rg, bg)
+        x, y, z = p
+        J = np.array([[f / z, 0, -f * x / z ** 2], [0, f / z, -f * y / z ** 2]])
+        S2 = J @ S3 @ J.T + 0.3 * np.eye(2)
+        assert abs(S2[0, 1]) > 0.2 * math.sqrt(S2[0, 0] * S2[1, 1])            # really tilted on the screen
+        Si = np.linalg.inv(S2)
+        cx, cy = f * x / z + (W - 1) / 2, f * y / z + (H - 1) / 2
+        ys, xs = np.mgrid[0:H, 0:W]
+        dx, dy = xs - cx, ys - cy
+        alpha = op * np.exp(-0.5 * (Si[0, 0] * dx * dx + 2 * Si[0, 1] * dx * dy + Si[1, 1] * dy * dy))
+        want = alpha[..., None] * np.array([0.9, 0.5, 0.2]) + (1 - alpha)[..., None] * bg
+        emitted = np.zeros((gy, gx), bool)
+        emitted.reshape(-1)[(ks >> 32).astype(np.int64)] = True
+        mask = np.kron(emitted, np.ones((16, 16), bool))
+        assert alpha[mask].max() > 0.5
+        np.testing.assert_allclose(img[mask], want[mask], atol=3e-4)
+        # outside the emitted tiles the splat is below the 1/255 threshold and the image is the background
+        assert alpha[~mask].max() < 1 / 255 + 1e-4
+        np.testing.assert_allclose(img[~mask], np.broadcast_to(bg, img.shape)[~mask], atol=1e-6)
 
 
 def test_blend_two_gaussians_order_matters(oracle):
