@@ -46,7 +46,8 @@ constexpr uint32_t kMaxTableIds = 1u << 20;
 // with its own counter, a workgroup appends to the list of its index modulo kListShards): one
 // shared counter would serialise thousands of atomic additions on one address.
 constexpr int kListShards = 32;
-constexpr int kListClasses = 3;
+constexpr int kListClasses = 4;
+static_assert(kListClasses * kListShards * 4 <= 512, "the list counters fit in the 512 bytes in front of the lists");
 
 struct Workspace {
     size_t alt_keys, alt_values, hist, chunk_sums, seg_start, seg_flags, seg_lists, total;
@@ -68,7 +69,8 @@ Workspace workspace_for(int n)
     w.seg_lists = w.seg_flags + kMaxTableIds / 8;
     // counters (kListClasses * kListShards words), then per class kListShards lists, each able to
     // hold every segment of its class
-    w.total = w.seg_lists + 512 + (size_t)kListShards * (((size_t)n / 512 + 2) + ((size_t)n / 1024 + 2) + ((size_t)n / 4096 + 2)) * 4;
+    w.total = w.seg_lists + 512 + (size_t)kListShards * (((size_t)n / 512 + 2) + ((size_t)n / 1024 + 2) + ((size_t)n / 4096 + 2) +
+                                                         ((size_t)n / 8192 + 2)) * 4;
     return w;
 }
 
@@ -720,7 +722,8 @@ __global__ __launch_bounds__(kWave) void segment_sort_wave_kernel(
     const int* __restrict__ seg_start, uint32_t* __restrict__ seg_flags,
     int list_max0, int list_max1, int list_max2,
     uint32_t* __restrict__ seg_counts, uint32_t* __restrict__ list0, uint32_t* __restrict__ list1,
-    uint32_t* __restrict__ list2, uint32_t list_cap0, uint32_t list_cap1, uint32_t list_cap2)
+    uint32_t* __restrict__ list2, uint32_t* __restrict__ list3,
+    uint32_t list_cap0, uint32_t list_cap1, uint32_t list_cap2, uint32_t list_cap3)
 {
     __shared__ uint32_t s_v[kT * kWave];
     const int lane = threadIdx.x;
@@ -737,8 +740,8 @@ __global__ __launch_bounds__(kWave) void segment_sort_wave_kernel(
     int len = 0;
     if (lane < kIds && mine < ids) len = seg_start[mine + 1] - seg_start[mine];
     // This launch sees every tile id once: it also lists the ids of the longer segments by class
-    // (lengths up to list_max0, list_max1, list_max2), so that those fewer, longer-running
-    // segments can be dealt out evenly by the launches that follow.
+    // (lengths up to list_max0, list_max1, list_max2, and everything longer), so that those
+    // fewer, longer-running segments can be dealt out evenly by the launches that follow.
     if (list0) {
         // neighbouring tiles tend to be equally busy: mix the index so that every list gets its share
         const uint32_t shard = (blockIdx.x ^ (blockIdx.x >> 5) ^ (blockIdx.x >> 10) ^ (blockIdx.x >> 15)) % kListShards;
@@ -748,6 +751,8 @@ __global__ __launch_bounds__(kWave) void segment_sort_wave_kernel(
             list1[(size_t)shard * list_cap1 + atomicAdd(&seg_counts[1 * kListShards + shard], 1u)] = mine;
         else if (len > list_max1 && len <= list_max2)
             list2[(size_t)shard * list_cap2 + atomicAdd(&seg_counts[2 * kListShards + shard], 1u)] = mine;
+        else if (len > list_max2)
+            list3[(size_t)shard * list_cap3 + atomicAdd(&seg_counts[3 * kListShards + shard], 1u)] = mine;
     }
     for (uint64_t todo = ballot(len > min_len && len <= kT * kWave); todo; todo &= todo - 1) {
         const uint32_t v = first_id + (uint32_t)(__ffsll((long long)todo) - 1);
@@ -800,11 +805,16 @@ __device__ __forceinline__ void sort_segment_general(uint64_t* __restrict__ keys
     __syncthreads();
 }
 
+// With a table of segment starts the first list_blocks workgroups take the listed segments (the
+// ones longer than min_len: neighbouring tiles tend to be equally crowded, so they are dealt out
+// one segment at a time, round-robin), the workgroups behind them look at 64 tile ids each for
+// shorter segments that were flagged.
 __global__ __launch_bounds__(kSortBlock) void segment_sort_general_kernel(
     uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
     uint64_t* __restrict__ alt_keys, uint32_t* __restrict__ alt_values,
     int n, uint32_t tile_mask, int min_len, uint32_t ids,
-    const int* __restrict__ seg_start, const uint32_t* __restrict__ seg_flags)
+    const int* __restrict__ seg_start, const uint32_t* __restrict__ seg_flags,
+    const uint32_t* __restrict__ list, const uint32_t* __restrict__ list_count, uint32_t list_cap, uint32_t list_blocks)
 {
     __shared__ uint32_t s_cnt[kSortWaves][kBins];
     __shared__ uint32_t s_wave_sum[kSortWaves];
@@ -840,13 +850,22 @@ __global__ __launch_bounds__(kSortBlock) void segment_sort_general_kernel(
         return;
     }
 
-    const uint32_t first_id = blockIdx.x * (uint32_t)kWave;
+    if (blockIdx.x < list_blocks) {
+        const uint32_t shard = blockIdx.x % kListShards;
+        const uint32_t count = list_count[shard];
+        for (uint32_t i = blockIdx.x / kListShards; i < count; i += list_blocks / kListShards) {
+            const uint32_t v = list[(size_t)shard * list_cap + i];
+            sort_segment_general(keys, values, alt_keys, alt_values, seg_start[v], seg_start[v + 1], s_cnt, s_wave_sum, &s_flag);
+        }
+        return;
+    }
+    const uint32_t first_id = (blockIdx.x - list_blocks) * (uint32_t)kWave;
     if (tid < kWave) {
         const uint32_t v = first_id + (uint32_t)lane;
         bool take = false;
         if (v < ids) {
             const int len = seg_start[v + 1] - seg_start[v];
-            take = len > min_len || (len > 1 && ((seg_flags[v >> 5] >> (v & 31)) & 1u));
+            take = len > 1 && len <= min_len && ((seg_flags[v >> 5] >> (v & 31)) & 1u);
         }
         const uint64_t m = ballot(take);
         if (lane == 0) s_match = m;
@@ -950,10 +969,12 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         uint64_t* ks = gaussian_keys_sorted;
         uint32_t* vs = gaussian_values_sorted;
         uint32_t* seg_counts = (uint32_t*)(list_sorting_space + ws.seg_lists);
-        const uint32_t cap_small = (uint32_t)(n / 512 + 2), cap_medium = (uint32_t)(n / 1024 + 2), cap_large = (uint32_t)(n / 4096 + 2);
+        const uint32_t cap_small = (uint32_t)(n / 512 + 2), cap_medium = (uint32_t)(n / 1024 + 2), cap_large = (uint32_t)(n / 4096 + 2),
+                       cap_long = (uint32_t)(n / 8192 + 2);
         uint32_t* list_small = seg_counts + 128;
         uint32_t* list_medium = list_small + (size_t)kListShards * cap_small;
         uint32_t* list_large = list_medium + (size_t)kListShards * cap_medium;
+        uint32_t* list_long = list_large + (size_t)kListShards * cap_large;
         const uint32_t* no_list = nullptr;
         // grids of the list-driven launches: a multiple of kListShards, enough for every listed segment
         auto list_grid = [](unsigned most, unsigned limit) {
@@ -976,12 +997,12 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
             hipLaunchKernelGGL((segment_sort_wave_kernel<kCapSmall / kWave, 1>), dim3(ids), dim3(kWave),
                                0, st, ks, vs, n, tile_mask, 1, ids, (const int*)seg_start, seg_flags,
                                kCapSmall, kCapMedium, kCapLarge, seg_counts, list_small, list_medium,
-                               list_large, cap_small, cap_medium, cap_large);
+                               list_large, list_long, cap_small, cap_medium, cap_large, cap_long);
         else
             hipLaunchKernelGGL((segment_sort_wave_kernel<kCapTiny / kWave, 1>), dim3(ids), dim3(kWave),
                                0, st, ks, vs, n, tile_mask, 1, ids, (const int*)seg_start, seg_flags,
                                kCapSmall, kCapMedium, kCapLarge, seg_counts, seg_start ? list_small : nullptr, list_medium,
-                               list_large, cap_small, cap_medium, cap_large);
+                               list_large, list_long, cap_small, cap_medium, cap_large, cap_long);
         if (seg_start) {
             if (n > kCapTiny && !one_wave_launch)       // 513..1024: the same network over 16 register slots, from the lists
                 hipLaunchKernelGGL((segment_sort_wave_list_kernel<kCapSmall / kWave>),
@@ -1001,9 +1022,12 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
             if (n > kCapMedium) FGS_SEGMENT_CLASS(16, kCapLarge, 64, kCapMedium, ids, no_list, no_list, 0u);
         }
 #undef FGS_SEGMENT_CLASS
-        hipLaunchKernelGGL(segment_sort_general_kernel, dim3(seg_start ? (ids + kWave - 1) / kWave : ids),
+        // longer segments from their list, one workgroup per segment; behind them the shorter ones that were flagged
+        const unsigned long_blocks = seg_start && n > kCapLarge ? list_grid((unsigned)(n / (kCapLarge + 1) + 1), 2048u) : 0u;
+        hipLaunchKernelGGL(segment_sort_general_kernel, dim3(seg_start ? long_blocks + (ids + kWave - 1) / kWave : ids),
                            dim3(kSortBlock), 0, st, ks, vs, alt_keys, alt_values, n, tile_mask, kCapLarge, ids,
-                           (const int*)seg_start, (const uint32_t*)seg_flags);
+                           (const int*)seg_start, (const uint32_t*)seg_flags,
+                           (const uint32_t*)list_long, (const uint32_t*)(seg_counts + 3 * kListShards), cap_long, long_blocks);
     }
     return check_hip(hipGetLastError(), "sort launch");
 }
