@@ -7,16 +7,20 @@ sort, tile ranges, blend - on a synthetic scene that is resident in HBM before t
 calls go through the C ABI of libflashgs_hip.so on torch's current HIP stream; the output image
 and every work buffer are allocated once, outside the timed region.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..4] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..4] [--no-cpu-baseline] [--headline-only]
 
-Prints one JSON line.  ``value`` is frames per second of the whole frame; ``roofline`` describes
-the dominant kernel (the blend), ``stages`` every stage with its algorithmic bytes against the
-8 TB/s HBM peak, ``cpu_baseline`` the same frame computed by the multithreaded CPU oracle on this
-machine's host cores.
+Prints one JSON line.  ``value`` is frames per second of the whole frame on the headline workload
+(``--config``, default the 4K / 3M one); ``roofline`` describes its dominant kernel (the blend),
+``stages`` every stage with its algorithmic bytes against the 8 TB/s HBM peak, ``cpu_baseline`` the
+same frame computed by the multithreaded CPU oracle on this machine's host cores,
+``ops_surface_ms_per_frame`` the same frame through ``flash_gaussian_splatting.ops`` the way
+``example.py:130-141`` times it, and ``configs`` the same figures for every other benchmark
+configuration (the 60-pose orbit at both frame sizes with per-frame p50 / p99).
 """
 import argparse
 import json
 import os
+import re
 import statistics
 import sys
 import time
@@ -28,11 +32,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3         # MI355X fp32 vector, published (packed FMA)
 LANE_SLOTS_PER_S = 256 * 4 * 16 * 2.4e9   # VALU issue slots per second without packed math
-# HBM bytes per blend launch on the headline configuration, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE scaled by the readings of a 256 MiB copy (profiles/frame_cfg2_4K_hbm_traffic.txt); other workloads: not measured
-BLEND_TRAFFIC_BYTES = {"cfg2_3M_4K": 1041157041}
 FLOP_PER_EVAL = 19               # render.cu:40-52: 2 sub, 6 mul + 3 add, 1 mul, 3 FMA, 1 sub
 SLOTS_PER_EVAL = 17              # 13 VALU with FMA contraction + a quarter-rate exp2 (the reference formulation)
+CAPACITY = {0: 1 << 20, 1: 1 << 22, 2: 1 << 24, 3: 1 << 25, 4: 1 << 25}
 
 
 def parse():
@@ -43,6 +45,8 @@ def parse():
     ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (default: the 4K / 3M headline)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-reps", type=int, default=3)
+    ap.add_argument("--headline-only", action="store_true", help="skip the other configurations (field \"configs\")")
+    ap.add_argument("--other-steps", type=int, default=20, help="timed frames per other configuration")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy, as the known-size reference for FETCH_SIZE / WRITE_SIZE")
     ap.add_argument("--size", default=None, metavar="WxH",
@@ -113,12 +117,204 @@ def cpu_baseline(sc, cam, capacity, reps):
         t4 = time.perf_counter()
         totals.append(t4 - t0)
         if per_stage is None or (t4 - t0) <= min(totals):
-            per_stage = dict(preprocess=(t1 - t0) * 1e3, sort=(t2 - t1) * 1e3, ranges=(t3 - t2) * 1e3, blend=(t4 - t3) * 1e3)
+            per_stage = dict(preprocess=round((t1 - t0) * 1e3, 2), sort=round((t2 - t1) * 1e3, 2),
+                             ranges=round((t3 - t2) * 1e3, 2), blend=round((t4 - t3) * 1e3, 2))
         counts = pre["counts"]
     med = statistics.median(totals)
-    return dict(value=1.0 / med, unit="frames/s", cores=threads, kind="port",
-                sample="%d full frame(s) of the benchmark workload, median" % len(totals),
-                ms_per_frame=med * 1e3, stages_ms=per_stage), counts, walked
+    return dict(value=round(1.0 / med, 3), unit="frames/s", cores=threads, kind="port",
+                sample="%d full frame(s) of this workload (first pose), median" % len(totals),
+                ms_per_frame=round(med * 1e3, 2), stages_ms=per_stage), counts, walked
+
+
+def profiled_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` on `workload` from the committed counter summary
+    profiles/frame_<workload>_hbm_traffic.txt (line "traffic_bytes <kernel>: <bytes>"), with the
+    summary's date; None where no summary covers it."""
+    path = os.path.join(ROOT, "profiles", "frame_%s_hbm_traffic.txt" % workload)
+    if not os.path.exists(path):
+        return None, None
+    text = open(path).read()
+    date = re.search(r"^measured: *(\S+)", text, re.M)
+    for m in re.finditer(r"^traffic_bytes +(.+?): *(\d+)", text, re.M):
+        if m.group(1).strip() == kernel:
+            return int(m.group(2)), "profiles/%s%s" % (os.path.basename(path), " (%s)" % date.group(1) if date else "")
+    return None, None
+
+
+class Frame:
+    """One configuration resident on the GPU with every buffer a frame needs."""
+
+    def __init__(self, torch, np, cabi, scenes, config, size=None):
+        kw = {}
+        if size:
+            kw["width"], kw["height"] = size
+        self.torch, self.np, self.cabi = torch, np, cabi
+        self.sc = scenes.make(config, **kw)
+        self.cams = self.sc.cameras
+        cam = self.cams[0]
+        self.W, self.H = cam.width, cam.height
+        self.n = n = self.sc.num_vertex
+        self.capacity = capacity = CAPACITY.get(config, 1 << 24)
+        dev = torch.device("cuda:0")
+        gx, gy = (self.W + 15) // 16, (self.H + 15) // 16
+        self.tiles = gx * gy
+
+        def up(a):
+            return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+        self.position, self.shs, self.opacity, self.cov3d = up(self.sc.position), up(self.sc.shs), up(self.sc.opacity), up(self.sc.cov3d)
+        self.points_xy = torch.zeros((n, 2), device=dev)
+        self.rgb_depth = torch.zeros((n, 4), device=dev)
+        self.conic_opacity = torch.zeros((n, 4), device=dev)
+        self.keys_u = torch.zeros(capacity, device=dev, dtype=torch.int64)
+        self.vals_u = torch.zeros(capacity, device=dev, dtype=torch.int32)
+        self.keys_s = torch.zeros(capacity, device=dev, dtype=torch.int64)
+        self.vals_s = torch.zeros(capacity, device=dev, dtype=torch.int32)
+        self.sort_size = cabi.get_sort_buffer_size(capacity)
+        self.sort_space = torch.zeros(self.sort_size, device=dev, dtype=torch.int8)
+        self.ranges = torch.zeros((self.tiles, 2), device=dev, dtype=torch.int32)
+        self.curr_offset = torch.zeros(1, device=dev, dtype=torch.int32)
+        self.offset_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        self.out_color = torch.zeros((self.H, self.W, 3), device=dev, dtype=torch.uint8)
+        self.bg = np.zeros(3, np.float32)
+        self.stream = torch.cuda.current_stream().cuda_stream
+        self.P = {k: getattr(self, k).data_ptr() for k in (
+            "position", "shs", "opacity", "cov3d", "points_xy", "rgb_depth", "conic_opacity", "keys_u", "vals_u",
+            "keys_s", "vals_s", "sort_space", "ranges", "curr_offset", "out_color")}
+
+    def frame(self, c, ev=None):
+        cabi, P, W, H, st = self.cabi, self.P, self.W, self.H, self.stream
+        if ev: ev[0].record()
+        self.curr_offset.zero_()
+        cabi.preprocess(self.n, P["position"], P["shs"], P["opacity"], P["cov3d"], W, H, 16, 16, c.position, c.rotation,
+                        c.focal_x, c.focal_y, c.zFar, c.zNear, P["points_xy"], P["rgb_depth"], P["conic_opacity"],
+                        P["keys_u"], P["vals_u"], P["curr_offset"], self.capacity, st)
+        if ev: ev[1].record()
+        self.offset_host.copy_(self.curr_offset)          # blocking read of the pair count (example.py:79)
+        K = int(self.offset_host[0])
+        if K < 0 or K >= self.capacity:
+            raise RuntimeError("too many pairs: %d (capacity %d)" % (K, self.capacity))
+        if ev: ev[2].record()
+        cabi.sort_gaussian(K, W, H, 16, 16, P["sort_space"], self.sort_size, P["keys_u"], P["vals_u"], P["keys_s"], P["vals_s"], st)
+        if ev: ev[3].record()
+        cabi.tile_ranges(16, 16, K, W, H, P["keys_s"], P["ranges"], st)
+        if ev: ev[4].record()
+        cabi.blend(16, 16, W, H, P["points_xy"], P["rgb_depth"], P["conic_opacity"], P["vals_s"], P["ranges"], self.bg,
+                   P["out_color"], None, st)
+        if ev: ev[5].record()
+        return K
+
+    def timed(self, cams, steps, warmup, per_frame_sync):
+        """steps frames over `cams` in turn: (ms per step, per-stage mean ms, per-frame ms or [], pair count of the first)."""
+        torch = self.torch
+        for i in range(warmup):
+            self.frame(cams[i % len(cams)])
+        torch.cuda.synchronize()
+        events = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(steps)]
+        frame_ms, Ks = [], []
+        torch.cuda.synchronize()
+        t_start = time.perf_counter()
+        for i in range(steps):
+            t0 = time.perf_counter()
+            Ks.append(self.frame(cams[i % len(cams)], events[i]))
+            if per_frame_sync:            # per-frame latency only matters for the trajectory workload
+                torch.cuda.synchronize()
+                frame_ms.append((time.perf_counter() - t0) * 1e3)
+        torch.cuda.synchronize()
+        t_end = time.perf_counter()
+        names = ["preprocess", "readback", "sort", "ranges", "blend"]
+        stage_ms = {nm: statistics.mean(ev[j].elapsed_time(ev[j + 1]) for ev in events) for j, nm in enumerate(names)}
+        return (t_end - t_start) * 1e3 / steps, stage_ms, frame_ms, Ks[0]
+
+
+def stage_report(fr, stage_ms, K, counts, walked):
+    """Per-stage figures against the rooflines that bound them, and the roofline block of the blend."""
+    n, W, H, tiles = fr.n, fr.W, fr.H, fr.tiles
+    passes = (32 + int(tiles).bit_length() + 7) // 8
+    stages = {}
+
+    def hbm(name, nbytes):
+        ms = stage_ms[name]
+        gbs = nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+        stages[name] = dict(ms=round(ms, 4), bound="hbm", algorithmic_bytes=int(nbytes),
+                            achieved_GBs=round(gbs, 1), peak_GBs=HBM_PEAK_GBS, frac=round(gbs / HBM_PEAK_GBS, 4))
+
+    if counts is not None:
+        hbm("preprocess", 16 * n + 24 * counts["n_pass"] + 232 * counts["visible"] + 12 * K)
+    else:
+        stages["preprocess"] = dict(ms=round(stage_ms["preprocess"], 4), bound="hbm")
+    hbm("sort", K * (8 + 24 * passes))
+    tile_passes = (int(tiles).bit_length() + 7) // 8
+    stages["sort"]["design_bytes"] = int(K * (32 * tile_passes + 8 + 24))   # count + scatter per tile digit, starts, segment sort
+    hbm("ranges", 8 * K + 16 * tiles)
+    stages["readback"] = dict(ms=round(stage_ms["readback"], 4), bound="host latency (4-byte read + sync)")
+
+    blend_ms = stage_ms["blend"]
+    kernel = fr.cabi.blend_kernel_name(16, 16, W, H)
+    traffic, source = profiled_traffic(fr.sc.name, kernel)
+    roofline = dict(kernel=kernel, bound="valu", achieved=None, peak=FP32_PEAK_TFLOPS, unit="TFLOP/s", frac=None,
+                    traffic=traffic, traffic_source=source, launch_ms=round(blend_ms, 4))
+    stages["blend"] = dict(ms=round(blend_ms, 4), bound="valu", kernel=kernel)
+    if walked is not None:
+        evals = 256 * walked
+        tflops = FLOP_PER_EVAL * evals / (blend_ms * 1e-3) / 1e12
+        roofline.update(achieved=round(tflops, 2), frac=round(tflops / FP32_PEAK_TFLOPS, 4),
+                        evaluations=int(evals), flop_per_evaluation=FLOP_PER_EVAL,
+                        # VALU issue slots the reference's formula would take (13 + 4 for exp2 per evaluation)
+                        # over the slots the chip has in that time: above 1, because the kernel gets the
+                        # exponent from tabulated parts (8.1 VALU instructions per evaluation measured)
+                        reference_formula_issue_slot_frac=round(SLOTS_PER_EVAL * evals / (blend_ms * 1e-3) / LANE_SLOTS_PER_S, 4),
+                        hbm_bytes=int(8 * tiles + 44 * walked + 3 * W * H))
+        stages["blend"].update(achieved_TFLOPs=roofline["achieved"], frac=roofline["frac"])
+    return stages, roofline
+
+
+def ops_surface_ms(torch, np, fr, steps):
+    """The same frame through flash_gaussian_splatting.ops, timed as example.py:130-141 does: one
+    untimed frame, then the mean over `steps` frames between two synchronisations."""
+    from flashgs_amd.rasterizer import Camera, Rasterizer, Scene
+    scene = Scene(torch.device("cuda:0"))
+    scene.num_vertex = fr.n
+    scene.position, scene.shs, scene.opacity, scene.cov3d = fr.position, fr.shs, fr.opacity, fr.cov3d
+    cam = Camera.from_synthetic(fr.cams[0])
+    rast = Rasterizer(scene, fr.capacity, fr.tiles, max_width=fr.W, max_height=fr.H)
+    bg = torch.zeros(3, dtype=torch.float32)
+    img = rast.forward(scene, cam, bg)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        img = rast.forward(scene, cam, bg)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    same = bool(torch.equal(img, fr.out_color))
+    del rast
+    return round(ms, 4), same
+
+
+def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops):
+    torch, np, cabi, scenes = mods
+    fr = Frame(torch, np, cabi, scenes, config, size)
+    ms_per_step, stage_ms, _, K = fr.timed(fr.cams[:1], steps, warmup, False)
+    cpu, counts, walked = (None, None, None)
+    if with_cpu:
+        cpu, counts, walked = cpu_baseline(fr.sc, fr.cams[0], fr.capacity, cpu_reps)
+    stages, roofline = stage_report(fr, stage_ms, K, counts, walked)
+    rep = dict(workload=fr.sc.name, gaussians=fr.n, width=fr.W, height=fr.H, pairs=int(K), poses=len(fr.cams),
+               ms_per_frame=round(ms_per_step, 4), fps=round(1000.0 / ms_per_step, 2), stages=stages, roofline=roofline,
+               cpu_baseline=cpu)
+    if counts is not None:
+        rep.update(n_pass=counts["n_pass"], visible=counts["visible"], walked=int(walked))
+    if len(fr.cams) > 1:
+        # the trajectory: every pose once, the per-frame pipeline re-run, host-timed with a sync per frame
+        traj_ms, traj_stage, frame_ms, _ = fr.timed(fr.cams, len(fr.cams), min(warmup, 3), True)
+        frame_ms.sort()
+        rep["trajectory"] = dict(poses=len(fr.cams), ms_per_frame_mean=round(traj_ms, 4),
+                                 frame_ms_p50=round(frame_ms[len(frame_ms) // 2], 4),
+                                 frame_ms_p99=round(frame_ms[min(len(frame_ms) - 1, int(0.99 * len(frame_ms)))], 4),
+                                 stages_ms_mean={k: round(v, 4) for k, v in traj_stage.items()})
+    if with_ops:
+        rep["ops_surface_ms_per_frame"], rep["ops_surface_image_identical"] = ops_surface_ms(torch, np, fr, steps)
+    return rep, fr
 
 
 def main():
@@ -137,68 +333,16 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
+    mods = (torch, np, cabi, scenes)
 
-    kw = {}
+    size = None
     if args.size:
         if args.config != 4:
             sys.exit("bench.py: --size applies to the trajectory workload (--config 4) only")
-        kw["width"], kw["height"] = (int(v) for v in args.size.lower().split("x"))
-    sc = scenes.make(args.config, **kw)
-    cams = sc.cameras
-    cam = cams[0]
-    W, H = cam.width, cam.height
-    n = sc.num_vertex
-    gx, gy = (W + 15) // 16, (H + 15) // 16
-    capacity = {0: 1 << 20, 1: 1 << 22, 2: 1 << 24, 3: 1 << 28, 4: 1 << 25}.get(args.config, 1 << 24)
+        size = tuple(int(v) for v in args.size.lower().split("x"))
+    with_cpu = not args.no_cpu_baseline
 
-    def up(a):
-        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
-
-    position, shs, opacity, cov3d = up(sc.position), up(sc.shs), up(sc.opacity), up(sc.cov3d)
-    points_xy = torch.zeros((n, 2), device=dev)
-    rgb_depth = torch.zeros((n, 4), device=dev)
-    conic_opacity = torch.zeros((n, 4), device=dev)
-    keys_u = torch.zeros(capacity, device=dev, dtype=torch.int64)
-    vals_u = torch.zeros(capacity, device=dev, dtype=torch.int32)
-    keys_s = torch.zeros(capacity, device=dev, dtype=torch.int64)
-    vals_s = torch.zeros(capacity, device=dev, dtype=torch.int32)
-    sort_size = cabi.get_sort_buffer_size(capacity)
-    sort_space = torch.zeros(sort_size, device=dev, dtype=torch.int8)
-    ranges = torch.zeros((gx * gy, 2), device=dev, dtype=torch.int32)
-    curr_offset = torch.zeros(1, device=dev, dtype=torch.int32)
-    offset_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
-    out_color = torch.zeros((H, W, 3), device=dev, dtype=torch.uint8)
-    bg = np.zeros(3, np.float32)
-    stream = torch.cuda.current_stream().cuda_stream
-    P = {k: v.data_ptr() for k, v in dict(position=position, shs=shs, opacity=opacity, cov3d=cov3d, points_xy=points_xy,
-                                          rgb_depth=rgb_depth, conic_opacity=conic_opacity, keys_u=keys_u, vals_u=vals_u,
-                                          keys_s=keys_s, vals_s=vals_s, sort_space=sort_space, ranges=ranges,
-                                          curr_offset=curr_offset, out_color=out_color).items()}
-
-    def frame(c, ev=None):
-        if ev: ev[0].record()
-        curr_offset.zero_()
-        cabi.preprocess(n, P["position"], P["shs"], P["opacity"], P["cov3d"], W, H, 16, 16, c.position, c.rotation,
-                        c.focal_x, c.focal_y, c.zFar, c.zNear, P["points_xy"], P["rgb_depth"], P["conic_opacity"],
-                        P["keys_u"], P["vals_u"], P["curr_offset"], capacity, stream)
-        if ev: ev[1].record()
-        offset_host.copy_(curr_offset)          # blocking read of the pair count (example.py:79)
-        K = int(offset_host[0])
-        if K < 0 or K >= capacity:
-            raise RuntimeError("too many pairs: %d (capacity %d)" % (K, capacity))
-        if ev: ev[2].record()
-        cabi.sort_gaussian(K, W, H, 16, 16, P["sort_space"], sort_size, P["keys_u"], P["vals_u"], P["keys_s"], P["vals_s"], stream)
-        if ev: ev[3].record()
-        cabi.tile_ranges(16, 16, K, W, H, P["keys_s"], P["ranges"], stream)
-        if ev: ev[4].record()
-        cabi.blend(16, 16, W, H, P["points_xy"], P["rgb_depth"], P["conic_opacity"], P["vals_s"], P["ranges"], bg,
-                   P["out_color"], None, stream)
-        if ev: ev[5].record()
-        return K
-
-    for i in range(args.warmup):
-        frame(cams[i % len(cams)])
-    torch.cuda.synchronize()
+    head, fr = run_config(mods, args.config, size, args.steps, args.warmup, args.cpu_reps, with_cpu, True)
     if args.copy_calibration:
         src = torch.ones(64 << 20, device=dev, dtype=torch.float32)      # 256 MiB read + 256 MiB written
         dst = torch.empty_like(src)
@@ -206,86 +350,43 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(args.steps)]
-    frame_ms, Ks = [], []
-    torch.cuda.synchronize()
-    t_start = time.perf_counter()
-    for i in range(args.steps):
-        t0 = time.perf_counter()
-        Ks.append(frame(cams[i % len(cams)], events[i]))
-        if len(cams) > 1:            # per-frame latency only matters for the trajectory workload
-            torch.cuda.synchronize()
-            frame_ms.append((time.perf_counter() - t0) * 1e3)
-    torch.cuda.synchronize()
-    t_end = time.perf_counter()
-    ms_per_step = (t_end - t_start) * 1e3 / args.steps
-    fps = 1000.0 / ms_per_step
-
-    names = ["preprocess", "readback", "sort", "ranges", "blend"]
-    stage_ms = {nm: statistics.mean(ev[j].elapsed_time(ev[j + 1]) for ev in events) for j, nm in enumerate(names)}
-    K = Ks[0]
-
-    cpu, counts, walked = (None, None, None)
-    if not args.no_cpu_baseline:
-        cpu, counts, walked = cpu_baseline(sc, cam, capacity, args.cpu_reps)
-
-    tiles = gx * gy
-    passes = (32 + int(tiles).bit_length() + 7) // 8
-    stages = {}
-
-    def hbm(name, nbytes):
-        ms = stage_ms[name]
-        gbs = nbytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
-        stages[name] = dict(ms=round(ms, 4), bound="hbm", algorithmic_bytes=int(nbytes),
-                            achieved_GBs=round(gbs, 1), peak_GBs=HBM_PEAK_GBS, frac=round(gbs / HBM_PEAK_GBS, 4))
-
-    if counts is not None and len(cams) == 1:
-        hbm("preprocess", 16 * n + 24 * counts["n_pass"] + 232 * counts["visible"] + 12 * K)
-    else:
-        stages["preprocess"] = dict(ms=round(stage_ms["preprocess"], 4), bound="hbm")
-    hbm("sort", K * (8 + 24 * passes))
-    tile_passes = (int(tiles).bit_length() + 7) // 8
-    stages["sort"]["design_bytes"] = int(K * (32 * tile_passes + 8 + 24))   # count + scatter per tile digit, starts, segment sort
-    hbm("ranges", 8 * K + 16 * tiles)
-    stages["readback"] = dict(ms=round(stage_ms["readback"], 4), bound="host latency (4-byte read + sync)")
-
-    blend_ms = stage_ms["blend"]
-    roofline = dict(kernel="blend_kernel_few_waves<1,1> (16x16 tile, one wave64, 2x2 pixels per lane)", bound="valu", achieved=None,
-                    peak=FP32_PEAK_TFLOPS, unit="TFLOP/s", frac=None, traffic=BLEND_TRAFFIC_BYTES.get(sc.name),
-                    launch_ms=round(blend_ms, 4))
-    if walked is not None and len(cams) == 1:
-        evals = 256 * walked
-        tflops = FLOP_PER_EVAL * evals / (blend_ms * 1e-3) / 1e12
-        roofline.update(achieved=round(tflops, 2), frac=round(tflops / FP32_PEAK_TFLOPS, 4),
-                        evaluations=int(evals), flop_per_evaluation=FLOP_PER_EVAL,
-                        # VALU issue slots the reference's formula would take (13 + 4 for exp2 per evaluation)
-                        # over the slots the chip has in that time: above 1, because the kernel gets the
-                        # exponent from tabulated parts (8.1 VALU instructions per evaluation measured)
-                        reference_formula_issue_slot_frac=round(SLOTS_PER_EVAL * evals / (blend_ms * 1e-3) / LANE_SLOTS_PER_S, 4),
-                        hbm_bytes=int(8 * tiles + 44 * walked + 3 * W * H))
-    stages["blend"] = dict(ms=round(blend_ms, 4), bound="valu")
-
     result = {
         "metric": "frames/s, full forward frame (preprocess + sort + ranges + blend)",
-        "value": round(fps, 2), "unit": "frames/s",
+        "value": head["fps"], "unit": "frames/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "ms_per_step": head["ms_per_frame"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": sc.name, "gaussians": n, "width": W, "height": H, "tile": "16x16",
-                   "sh_degree": 3, "pairs": int(K), "poses": len(cams)},
+        "config": {"workload": head["workload"], "gaussians": head["gaussians"], "width": head["width"], "height": head["height"],
+                   "tile": "16x16", "sh_degree": 3, "pairs": head["pairs"], "poses": head["poses"]},
         "target_fps": 400 if args.config == 2 else None,
-        "stages": stages,
-        "roofline": roofline,
-        "cpu_baseline": cpu,
+        "stages": head["stages"],
+        "roofline": head["roofline"],
+        "cpu_baseline": head["cpu_baseline"],
+        "ops_surface_ms_per_frame": head["ops_surface_ms_per_frame"],
+        "ops_surface_image_identical": head["ops_surface_image_identical"],
     }
-    if counts is not None:
-        result["config"].update(n_pass=counts["n_pass"], visible=counts["visible"], walked=int(walked))
-    if frame_ms:
-        frame_ms.sort()
-        result["frame_ms_p50"] = round(frame_ms[len(frame_ms) // 2], 4)
-        result["frame_ms_p99"] = round(frame_ms[min(len(frame_ms) - 1, int(0.99 * len(frame_ms)))], 4)
+    for k in ("n_pass", "visible", "walked"):
+        if k in head:
+            result["config"][k] = head[k]
+    if "trajectory" in head:
+        result["trajectory"] = head["trajectory"]
+        result["frame_ms_p50"] = head["trajectory"]["frame_ms_p50"]
+        result["frame_ms_p99"] = head["trajectory"]["frame_ms_p99"]
     if args.calibrate:
         result["calibration"] = calibrate(torch, dev)
+    del fr
+    torch.cuda.empty_cache()
+
+    if not args.headline_only:
+        others = {}
+        for config, sz in ((0, None), (1, None), (2, None), (3, None), (4, None), (4, (3840, 2160))):
+            if config == args.config and sz == size:
+                continue
+            rep, fr_o = run_config(mods, config, sz, args.other_steps, min(args.warmup, 3), 1, with_cpu, False)
+            others[rep["workload"]] = rep
+            del fr_o
+            torch.cuda.empty_cache()
+        result["configs"] = others
     print(json.dumps(result))
 
 

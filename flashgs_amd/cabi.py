@@ -30,6 +30,7 @@ SIGNATURES = {
     "fgs_render_f32": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 9 + [C.c_void_p]),
     "fgs_tile_ranges": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 3),
     "fgs_blend": (C.c_int, [C.c_int] * 4 + [C.c_void_p] * 9),
+    "fgs_blend_kernel_name": (C.c_char_p, [C.c_int] * 4),
     "fgs_camera_matrices": (None, [C.c_void_p] * 2 + [C.c_int] * 2 + [C.c_float] * 4 + [C.c_void_p] * 2),
     "fgs_set_scan_spin_limit": (C.c_uint, [C.c_uint]),
     "fgs_last_error": (C.c_char_p, []),
@@ -125,6 +126,11 @@ def render_f32(block_x, block_y, num_rendered, width, height, points_xy, rgb_dep
     rc = load().fgs_render_f32(block_x, block_y, num_rendered, width, height, points_xy, rgb_depth, conic_opacity,
                                keys_sorted, values_sorted, ranges, bg.ctypes.data, out_u8, out_f32, stream)
     _check(rc, "fgs_render_f32")
+
+
+def blend_kernel_name(block_x, block_y, width, height):
+    """The kernel(s) a blend of this tile and frame size launches on the current device."""
+    return load().fgs_blend_kernel_name(block_x, block_y, width, height).decode()
 
 
 def tile_ranges(block_x, block_y, num_rendered, width, height, keys_sorted, ranges, stream=0):

@@ -762,6 +762,19 @@ extern "C" int fgs_render_f32(int block_x, int block_y, int num_rendered, int wi
                             out_color_u8, out_color_f32, stream, "fgs_render_f32");
 }
 
+extern "C" const char* fgs_blend_kernel_name(int block_x, int block_y, int width, int height)
+{
+    using namespace fgs;
+    int sx = 0, sy = 0;
+    if (check_tile(block_x, block_y, &sx, &sy, "fgs_blend_kernel_name") != FGS_OK || width <= 0 || height <= 0) return "";
+    BlendShape shape;
+    if (blend_shape(block_x, block_y, (width + block_x - 1) / block_x, (height + block_y - 1) / block_y, &shape) != FGS_OK) return "";
+    if (shape.shared) return "tile_order_kernel + blend_kernel_shared";
+    if (sx == 1 && sy == 1) return shape.few_waves ? "blend_kernel_few_waves<1, 1>" : "blend_kernel<1, 1>";
+    if (sx == 2 && sy == 1) return shape.few_waves ? "blend_kernel_few_waves<2, 1>" : "blend_kernel<2, 1>";
+    return shape.few_waves ? "blend_kernel_few_waves<2, 2>" : "blend_kernel<2, 2>";
+}
+
 extern "C" int fgs_tile_ranges(int block_x, int block_y, int num_rendered, int width, int height,
                                const uint64_t* gaussian_keys_sorted, int* ranges, void* stream)
 {

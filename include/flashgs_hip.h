@@ -156,6 +156,14 @@ int fgs_blend(int block_x, int block_y, int width, int height,
               uint8_t* out_color_u8, float* out_color_f32, void* stream);
 
 /*
+ * No counterpart in the reference.  Name of the kernel(s) fgs_blend / fgs_render_* launch on the
+ * current device for this tile and frame size (the choice depends on how many tiles the frame has
+ * against what the chip holds at once), as a profiler lists them; "" for an unsupported tile size.
+ * Lets a benchmark attribute its figures to the kernel that ran.
+ */
+const char* fgs_blend_kernel_name(int block_x, int block_y, int width, int height);
+
+/*
  * Host-side camera set-up used by fgs_preprocess (preprocess.cu:420-448,461-466), exposed so
  * callers and tests can inspect it: column-major 4x4 view and projection matrices.
  */
