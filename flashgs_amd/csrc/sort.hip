@@ -7,8 +7,9 @@
 // contiguous and ordered by depth.  So the sort runs most-significant part first:
 //
 //  1. Partition by tile id: one stable counting pass per 8 bits of tile id (two passes for up to
-//     65536 tiles).  A pass is count -> offsets -> scatter: `count_kernel` builds one digit
-//     histogram per block of 4096 pairs, `chunk_sum_kernel` + `offsets_kernel` turn the
+//     65536 tiles; above that digits of 9 bits, so an 8K frame of 129 600 tiles still takes two).
+//     A pass is count -> offsets -> scatter: `count_kernel` builds one digit
+//     histogram per block of 4096 pairs (3840 with 9-bit digits), `chunk_sum_kernel` + `offsets_kernel` turn the
 //     histograms into the exclusive start of every (block, digit) run, and `scatter_kernel` ranks
 //     its block in LDS (wave64 ballot matching, so equal digits keep their input order) and
 //     writes each run to its start.  No workgroup ever waits for another one.
@@ -29,12 +30,27 @@
 namespace fgs {
 namespace {
 
-constexpr int kBins = 256;
+constexpr int kBins = 256;                      // counters of a counting pass inside a segment (8-bit digits)
 constexpr int kSortBlock = 256;
 constexpr int kSortWaves = kSortBlock / kWave;
-constexpr int kItems = 16;                      // pairs per thread in count/scatter
-constexpr int kTile = kSortBlock * kItems;      // pairs per count/scatter workgroup
 constexpr int kMinChunk = 16;                   // fewest histogram rows summed by one chunk_sum workgroup
+
+// Shape of a partition pass: digits of kBitsT bits, kItemsT pairs per thread.  Up to 65 536 tiles
+// two passes of 8 bits do; above that (an 8K frame has 129 600) digits of 9 bits keep it at two
+// passes up to 262 144 tiles, with 15 pairs per thread so that the workgroup's LDS still lets
+// three workgroups share a CU.
+template <int kBitsT, int kItemsT>
+struct PassShape {
+    static constexpr int kBits = kBitsT;
+    static constexpr int kBinsP = 1 << kBitsT;
+    static constexpr int kItems = kItemsT;                  // pairs per thread in count/scatter
+    static constexpr int kTile = kSortBlock * kItemsT;      // pairs per count/scatter workgroup
+    static constexpr int kPerThread = kBinsP / kSortBlock;  // digits per thread where a thread stands for digits
+    static_assert(kBinsP % kSortBlock == 0 && kTile <= 65535, "16-bit counts per wave and digit");
+};
+using Narrow = PassShape<8, 16>;
+using Wide = PassShape<9, 15>;
+constexpr int kNarrowMaxTileBits = 16;
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -51,20 +67,35 @@ static_assert(kListClasses * kListShards * 4 <= 512, "the list counters fit in t
 
 struct Workspace {
     size_t alt_keys, alt_values, hist, chunk_sums, seg_start, seg_flags, seg_lists, total;
-    int tiles, chunk, chunks;       // chunks of `chunk` histogram rows each
 };
 
+struct PassGrid {
+    int tiles, chunk, chunks;       // workgroups of a count/scatter launch; chunks of `chunk` histogram rows each
+};
+
+PassGrid pass_grid(int n, int tile)
+{
+    PassGrid g;
+    g.tiles = (n + tile - 1) / tile;
+    g.chunk = (g.tiles + 255) / 256 > kMinChunk ? (g.tiles + 255) / 256 : kMinChunk;     // at most ~256 chunks
+    g.chunks = (g.tiles + g.chunk - 1) / g.chunk;
+    return g;
+}
+
+// Sized for whichever pass shape the frame turns out to need (the tile count is not known here).
 Workspace workspace_for(int n)
 {
     Workspace w;
-    w.tiles = (n + kTile - 1) / kTile;
-    w.chunk = (w.tiles + 255) / 256 > kMinChunk ? (w.tiles + 255) / 256 : kMinChunk;     // at most ~256 chunks
-    w.chunks = (w.tiles + w.chunk - 1) / w.chunk;
+    const PassGrid a = pass_grid(n, Narrow::kTile), b = pass_grid(n, Wide::kTile);
+    const size_t hist = (size_t)a.tiles * Narrow::kBinsP > (size_t)b.tiles * Wide::kBinsP ? (size_t)a.tiles * Narrow::kBinsP
+                                                                                           : (size_t)b.tiles * Wide::kBinsP;
+    const size_t sums = (size_t)a.chunks * Narrow::kBinsP > (size_t)b.chunks * Wide::kBinsP ? (size_t)a.chunks * Narrow::kBinsP
+                                                                                             : (size_t)b.chunks * Wide::kBinsP;
     w.alt_keys = 0;
     w.alt_values = align_up((size_t)n * 8, 256);
     w.hist = w.alt_values + align_up((size_t)n * 4, 256);
-    w.chunk_sums = w.hist + (size_t)w.tiles * kBins * 4;
-    w.seg_start = w.chunk_sums + (size_t)w.chunks * kBins * 4;
+    w.chunk_sums = w.hist + hist * 4;
+    w.seg_start = align_up(w.chunk_sums + sums * 4, 256);
     w.seg_flags = w.seg_start + align_up(((size_t)kMaxTableIds + 1) * 4, 256);
     w.seg_lists = w.seg_flags + kMaxTableIds / 8;
     // counters (kListClasses * kListShards words), then per class kListShards lists, each able to
@@ -81,56 +112,66 @@ __device__ __forceinline__ uint32_t digit_of(uint64_t key, int shift, uint32_t m
 
 // ---- partition pass, step 1: hist[block][digit] ---------------------------------------------------
 
+template <class Shape>
 __global__ __launch_bounds__(kSortBlock) void count_kernel(const uint64_t* __restrict__ keys, int n,
                                                            int shift, int nbits, uint32_t* __restrict__ hist)
 {
-    __shared__ uint32_t h[kBins];
+    constexpr int kB = Shape::kBinsP;
+    __shared__ uint32_t h[kB];
     const int tid = threadIdx.x;
-    h[tid] = 0;
+#pragma unroll
+    for (int q = 0; q < Shape::kPerThread; q++) h[q * kSortBlock + tid] = 0;
     __syncthreads();
     const uint32_t mask = (1u << nbits) - 1u;
-    const int base = blockIdx.x * kTile;
+    const int base = blockIdx.x * Shape::kTile;
 #pragma unroll
-    for (int i = 0; i < kItems; i++) {
+    for (int i = 0; i < Shape::kItems; i++) {
         const int idx = base + i * kSortBlock + tid;
         if (idx < n) atomicAdd(&h[digit_of(keys[idx], shift, mask)], 1u);
     }
     __syncthreads();
-    hist[(size_t)blockIdx.x * kBins + tid] = h[tid];
+#pragma unroll
+    for (int q = 0; q < Shape::kPerThread; q++)
+        hist[(size_t)blockIdx.x * kB + q * kSortBlock + tid] = h[q * kSortBlock + tid];
 }
 
 // ---- step 2: exclusive start of every (block, digit) run ----------------------------------------
 // start[b][d] = sum of hist[*][d' < d] + sum of hist[b' < b][d]   (digit-major, then block)
 
-__global__ __launch_bounds__(kBins) void chunk_sum_kernel(const uint32_t* __restrict__ hist, int tiles, int chunk,
-                                                          uint32_t* __restrict__ chunk_sums)
+template <class Shape>
+__global__ __launch_bounds__(Shape::kBinsP) void chunk_sum_kernel(const uint32_t* __restrict__ hist, int tiles, int chunk,
+                                                                  uint32_t* __restrict__ chunk_sums)
 {
+    constexpr int kB = Shape::kBinsP;
     const int d = threadIdx.x;
     const int t0 = blockIdx.x * chunk, t1 = min(tiles, t0 + chunk);
     uint32_t s = 0;
-    for (int t = t0; t < t1; t++) s += hist[(size_t)t * kBins + d];
-    chunk_sums[(size_t)blockIdx.x * kBins + d] = s;
+    for (int t = t0; t < t1; t++) s += hist[(size_t)t * kB + d];
+    chunk_sums[(size_t)blockIdx.x * kB + d] = s;
 }
 
-// One workgroup per chunk, up to kOffsetGroups threads per digit (blockDim.x / kBins of them): the
-// chunk sums are few and the loop over them is latency-bound, so each group of kBins threads
+// One workgroup per chunk, up to 1024 / bins threads per digit (blockDim.x / bins of them): the
+// chunk sums are few and the loop over them is latency-bound, so each group of `bins` threads
 // takes every groups-th batch of 16 independent loads.
-constexpr int kOffsetGroups = 4;
+constexpr int kOffsetThreads = 1024;
 
-__global__ __launch_bounds__(kBins * kOffsetGroups) void offsets_kernel(uint32_t* __restrict__ hist, int tiles, int chunk,
-                                                                        const uint32_t* __restrict__ chunk_sums, int chunks)
+template <class Shape>
+__global__ __launch_bounds__(kOffsetThreads) void offsets_kernel(uint32_t* __restrict__ hist, int tiles, int chunk,
+                                                                 const uint32_t* __restrict__ chunk_sums, int chunks)
 {
-    __shared__ uint32_t s_total[kOffsetGroups][kBins], s_before[kOffsetGroups][kBins];
-    __shared__ uint32_t s_wave[kBins / kWave];
-    const int d = threadIdx.x & (kBins - 1), group = threadIdx.x / kBins;
+    constexpr int kB = Shape::kBinsP;
+    constexpr int kMaxGroups = kOffsetThreads / kB;
+    __shared__ uint32_t s_total[kMaxGroups][kB], s_before[kMaxGroups][kB];
+    __shared__ uint32_t s_wave[kB / kWave];
+    const int d = threadIdx.x & (kB - 1), group = threadIdx.x / kB;
     const int lane = d & (kWave - 1), wave = d / kWave;
     const int mine = (int)blockIdx.x;
-    const int groups = (int)blockDim.x / kBins;
+    const int groups = (int)blockDim.x / kB;
     uint32_t total = 0, before = 0;
     for (int c0 = group * 16; c0 < chunks; c0 += 16 * groups) {
         uint32_t v[16];
 #pragma unroll
-        for (int j = 0; j < 16; j++) v[j] = c0 + j < chunks ? chunk_sums[(size_t)(c0 + j) * kBins + d] : 0u;
+        for (int j = 0; j < 16; j++) v[j] = c0 + j < chunks ? chunk_sums[(size_t)(c0 + j) * kB + d] : 0u;
 #pragma unroll
         for (int j = 0; j < 16; j++) {
             if (c0 + j < mine) before += v[j];
@@ -142,9 +183,9 @@ __global__ __launch_bounds__(kBins * kOffsetGroups) void offsets_kernel(uint32_t
     __syncthreads();
     total = 0; before = 0;
 #pragma unroll
-    for (int g = 0; g < kOffsetGroups; g++)
+    for (int g = 0; g < kMaxGroups; g++)
         if (g < groups) { total += s_total[g][d]; before += s_before[g][d]; }
-    // exclusive scan of the digit totals over the 256 digits (every group does the same sums)
+    // exclusive scan of the digit totals over the digits (every group does the same sums)
     uint32_t incl = wave_inclusive_sum(total);
     if (group == 0 && lane == kWave - 1) s_wave[wave] = incl;
     __syncthreads();
@@ -157,10 +198,10 @@ __global__ __launch_bounds__(kBins * kOffsetGroups) void offsets_kernel(uint32_t
     for (int tb = t0; tb < t1; tb += 16) {
         uint32_t c[16];
 #pragma unroll
-        for (int j = 0; j < 16; j++) c[j] = tb + j < t1 ? hist[(size_t)(tb + j) * kBins + d] : 0u;
+        for (int j = 0; j < 16; j++) c[j] = tb + j < t1 ? hist[(size_t)(tb + j) * kB + d] : 0u;
 #pragma unroll
         for (int j = 0; j < 16; j++) {
-            if (tb + j < t1) hist[(size_t)(tb + j) * kBins + d] = run;
+            if (tb + j < t1) hist[(size_t)(tb + j) * kB + d] = run;
             run += c[j];
         }
     }
@@ -170,14 +211,16 @@ __global__ __launch_bounds__(kBins * kOffsetGroups) void offsets_kernel(uint32_t
 // digit, no chunk sums in between.
 constexpr int kSmallRows = 64;
 
-__global__ __launch_bounds__(kBins) void offsets_small_kernel(uint32_t* __restrict__ hist, int tiles)
+template <class Shape>
+__global__ __launch_bounds__(Shape::kBinsP) void offsets_small_kernel(uint32_t* __restrict__ hist, int tiles)
 {
-    __shared__ uint32_t s_wave[kBins / kWave];
+    constexpr int kB = Shape::kBinsP;
+    __shared__ uint32_t s_wave[kB / kWave];
     const int d = threadIdx.x;
     const int lane = d & (kWave - 1), wave = d / kWave;
     uint32_t c[kSmallRows];
 #pragma unroll
-    for (int t = 0; t < kSmallRows; t++) c[t] = t < tiles ? hist[(size_t)t * kBins + d] : 0u;
+    for (int t = 0; t < kSmallRows; t++) c[t] = t < tiles ? hist[(size_t)t * kB + d] : 0u;
     uint32_t total = 0;
 #pragma unroll
     for (int t = 0; t < kSmallRows; t++) total += c[t];
@@ -188,26 +231,27 @@ __global__ __launch_bounds__(kBins) void offsets_small_kernel(uint32_t* __restri
     for (int w = 0; w < wave; w++) run += s_wave[w];
 #pragma unroll
     for (int t = 0; t < kSmallRows; t++) {
-        if (t < tiles) hist[(size_t)t * kBins + d] = run;
+        if (t < tiles) hist[(size_t)t * kB + d] = run;
         run += c[t];
     }
 }
 
 // ---- step 3: stable scatter ---------------------------------------------------------------------------
 
+template <class Shape>
 __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
     const uint64_t* __restrict__ keys_in, const uint32_t* __restrict__ values_in,
     uint64_t* __restrict__ keys_out, uint32_t* __restrict__ values_out,
     int n, int shift, int nbits,
-    const uint32_t* __restrict__ start)          // [blocks][kBins] from offsets_kernel
+    const uint32_t* __restrict__ start)          // [blocks][bins] from offsets_kernel
 {
+    constexpr int kB = Shape::kBinsP, kItems = Shape::kItems, kTile = Shape::kTile, kPer = Shape::kPerThread;
     // per-wave digit counts, then per-wave digit offsets: at most kTile, so 16 bits do, and with
     // them the workgroup's LDS stays under a third of the CU's (three resident workgroups, not two)
-    __shared__ uint16_t s_count[kSortWaves][kBins];
-    static_assert(kTile <= 65535, "s_count holds 16-bit counts");
-    __shared__ uint32_t s_bin_start[kBins];           // where each digit starts in the ranked block
-    __shared__ uint32_t s_global[kBins];              // destination of ranked slot p with digit d: s_global[d] + p
-    __shared__ uint32_t s_wave_sum[kSortWaves];
+    __shared__ uint16_t s_count[kSortWaves][kB];
+    __shared__ uint16_t s_bin_start[kB];              // where each digit starts in the ranked block
+    __shared__ uint32_t s_global[kB];                 // destination of ranked slot p with digit d: s_global[d] + p
+    __shared__ uint32_t s_wave_sum[kPer * kSortWaves];
     __shared__ uint64_t s_keys[kTile];
     __shared__ uint32_t s_values[kTile];
 
@@ -234,9 +278,13 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
         const int off = wave * (kWave * kItems) + i * kWave + lane;
         val[i] = off < in_tile ? values_in[tile_base + off] : 0u;
     }
-    const uint32_t my_start = start[(size_t)tile * kBins + tid];
+    uint32_t my_start[kPer];
 #pragma unroll
-    for (int w = 0; w < kSortWaves; w++) s_count[w][tid] = 0;
+    for (int q = 0; q < kPer; q++) my_start[q] = start[(size_t)tile * kB + q * kSortBlock + tid];
+#pragma unroll
+    for (int w = 0; w < kSortWaves; w++)
+#pragma unroll
+        for (int q = 0; q < kPer; q++) s_count[w][q * kSortBlock + tid] = 0;
     __syncthreads();
 
     // rank inside the wave: lanes with equal digits find each other with one ballot per digit bit
@@ -247,7 +295,7 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
         const uint32_t d = digit_of(key[i], shift, mask);
         uint64_t peers = ballot(valid);
 #pragma unroll
-        for (int b = 0; b < 8; b++) {
+        for (int b = 0; b < Shape::kBits; b++) {
             const bool bit = (d >> b) & 1u;
             const uint64_t with_bit = ballot(bit);
             peers &= bit ? with_bit : ~with_bit;
@@ -265,25 +313,34 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
     }
     __syncthreads();
 
-    // digit totals of the block; per-wave offsets inside each digit
-    const int d = tid;      // one thread per digit from here on
-    uint32_t total = 0;
+    // digit totals of the block; per-wave offsets inside each digit.  A thread stands for the
+    // digits tid, tid + 256, ...; the scan runs over the digits in their order.
+    uint32_t total[kPer], incl[kPer];
 #pragma unroll
-    for (int w = 0; w < kSortWaves; w++) {
-        const uint32_t c = s_count[w][d];
-        s_count[w][d] = (uint16_t)total;
-        total += c;
+    for (int q = 0; q < kPer; q++) {
+        const int d = q * kSortBlock + tid;
+        total[q] = 0;
+#pragma unroll
+        for (int w = 0; w < kSortWaves; w++) {
+            const uint32_t c = s_count[w][d];
+            s_count[w][d] = (uint16_t)total[q];
+            total[q] += c;
+        }
+        incl[q] = wave_inclusive_sum(total[q]);
+        if (lane == kWave - 1) s_wave_sum[q * kSortWaves + wave] = incl[q];
     }
-    uint32_t incl = wave_inclusive_sum(total);
-    if (lane == kWave - 1) s_wave_sum[wave] = incl;
     __syncthreads();
-    uint32_t before_wave = 0;
 #pragma unroll
-    for (int w = 0; w < kSortWaves; w++)
-        if (w < wave) before_wave += s_wave_sum[w];
-    const uint32_t bin_start = before_wave + incl - total;
-    s_bin_start[d] = bin_start;
-    s_global[d] = my_start - bin_start;
+    for (int q = 0; q < kPer; q++) {
+        const int d = q * kSortBlock + tid;
+        uint32_t before_wave = 0;
+#pragma unroll
+        for (int w = 0; w < kPer * kSortWaves; w++)
+            if (w < q * kSortWaves + wave) before_wave += s_wave_sum[w];
+        const uint32_t bin_start = before_wave + incl[q] - total[q];
+        s_bin_start[d] = (uint16_t)bin_start;
+        s_global[d] = my_start[q] - bin_start;
+    }
     __syncthreads();
 
     // move the pairs to their ranked slots in LDS
@@ -292,7 +349,7 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
         const int off = wave * (kWave * kItems) + i * kWave + lane;
         if (off < in_tile) {
             const uint32_t dg = digit_of(key[i], shift, mask);
-            const uint32_t p = s_bin_start[dg] + s_count[wave][dg] + slot[i];
+            const uint32_t p = (uint32_t)s_bin_start[dg] + s_count[wave][dg] + slot[i];
             s_keys[p] = key[i];
             s_values[p] = val[i];
         }
@@ -923,7 +980,6 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
     if (tiles_xy >= (1LL << 30)) return fail(FGS_E_INVALID, "fgs_sort_gaussian: too many tiles");
     const int tile_bits = bit_length((uint32_t)tiles_xy);         // sort.cu:34-39: bits [0, 32 + tile_bits)
     const uint32_t tile_mask = (1u << tile_bits) - 1u;
-    const int passes = (tile_bits + 7) / 8;
 
     hipStream_t st = (hipStream_t)stream;
     uint64_t* alt_keys = (uint64_t*)(list_sorting_space + ws.alt_keys);
@@ -932,26 +988,34 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
     uint32_t* chunk_sums = (uint32_t*)(list_sorting_space + ws.chunk_sums);
 
     // 1. stable partition by tile id, least significant tile digit first
-    const uint64_t* src_k = gaussian_keys_unsorted;
-    const uint32_t* src_v = gaussian_values_unsorted;
-    for (int p = 0; p < passes; p++) {
-        const bool to_sorted = ((passes - p) & 1) != 0;      // the last pass lands in the caller's sorted buffers
-        uint64_t* dst_k = to_sorted ? gaussian_keys_sorted : alt_keys;
-        uint32_t* dst_v = to_sorted ? gaussian_values_sorted : alt_values;
-        const int shift = 32 + 8 * p;
-        const int nbits = tile_bits - 8 * p < 8 ? tile_bits - 8 * p : 8;
-        hipLaunchKernelGGL(count_kernel, dim3(ws.tiles), dim3(kSortBlock), 0, st, src_k, n, shift, nbits, hist);
-        if (ws.tiles <= kSmallRows) {
-            hipLaunchKernelGGL(offsets_small_kernel, dim3(1), dim3(kBins), 0, st, hist, ws.tiles);
-        } else {
-            hipLaunchKernelGGL(chunk_sum_kernel, dim3(ws.chunks), dim3(kBins), 0, st, hist, ws.tiles, ws.chunk, chunk_sums);
-            hipLaunchKernelGGL(offsets_kernel, dim3(ws.chunks), dim3(kBins * (ws.chunks > 16 ? kOffsetGroups : 1)), 0, st, hist, ws.tiles, ws.chunk, chunk_sums, ws.chunks);
+    auto partition = [&](auto shape) {
+        using Shape = decltype(shape);
+        const PassGrid g = pass_grid(n, Shape::kTile);
+        const int passes = (tile_bits + Shape::kBits - 1) / Shape::kBits;
+        const uint64_t* src_k = gaussian_keys_unsorted;
+        const uint32_t* src_v = gaussian_values_unsorted;
+        for (int p = 0; p < passes; p++) {
+            const bool to_sorted = ((passes - p) & 1) != 0;      // the last pass lands in the caller's sorted buffers
+            uint64_t* dst_k = to_sorted ? gaussian_keys_sorted : alt_keys;
+            uint32_t* dst_v = to_sorted ? gaussian_values_sorted : alt_values;
+            const int shift = 32 + Shape::kBits * p;
+            const int nbits = tile_bits - Shape::kBits * p < Shape::kBits ? tile_bits - Shape::kBits * p : Shape::kBits;
+            hipLaunchKernelGGL((count_kernel<Shape>), dim3(g.tiles), dim3(kSortBlock), 0, st, src_k, n, shift, nbits, hist);
+            if (g.tiles <= kSmallRows) {
+                hipLaunchKernelGGL((offsets_small_kernel<Shape>), dim3(1), dim3(Shape::kBinsP), 0, st, hist, g.tiles);
+            } else {
+                hipLaunchKernelGGL((chunk_sum_kernel<Shape>), dim3(g.chunks), dim3(Shape::kBinsP), 0, st, hist, g.tiles, g.chunk, chunk_sums);
+                hipLaunchKernelGGL((offsets_kernel<Shape>), dim3(g.chunks), dim3(g.chunks > 16 ? kOffsetThreads : Shape::kBinsP), 0, st,
+                                   hist, g.tiles, g.chunk, chunk_sums, g.chunks);
+            }
+            hipLaunchKernelGGL((scatter_kernel<Shape>), dim3(g.tiles), dim3(kSortBlock), 0, st,
+                               src_k, src_v, dst_k, dst_v, n, shift, nbits, hist);
+            src_k = dst_k;
+            src_v = dst_v;
         }
-        hipLaunchKernelGGL(scatter_kernel, dim3(ws.tiles), dim3(kSortBlock), 0, st,
-                           src_k, src_v, dst_k, dst_v, n, shift, nbits, hist);
-        src_k = dst_k;
-        src_v = dst_v;
-    }
+    };
+    if (tile_bits <= kNarrowMaxTileBits) partition(Narrow());
+    else partition(Wide());
 
     // 2. every tile id's segment by depth, in place in the sorted buffers
     if (n > 1) {

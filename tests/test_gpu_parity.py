@@ -361,8 +361,8 @@ def test_sort_sizes_against_numpy(n):
     assert np.array_equal(gp.u32(vs)[:n], vals[order])
 
 
-def test_sort_8k_frame_three_partition_passes():
-    """7680x4320 has 129 600 tiles: 17 tile bits, three partition passes.  Against numpy."""
+def test_sort_8k_frame_wide_partition_digits():
+    """7680x4320 has 129 600 tiles: 17 tile bits, partitioned in two passes of 9-bit digits.  Against numpy."""
     rng = np.random.default_rng(8)
     n = 1_200_000
     tile = rng.integers(0, 480 * 270, n).astype(np.uint32)
@@ -523,8 +523,8 @@ def config3_scene():
 
 
 def test_config3_8k_frame(oracle, config3_scene):
-    """8M Gaussians at 7680x4320 (129 600 tiles, three partition passes, the blend variant with
-    fewer resident waves), 2 % of the splats enlarged: the whole frame against the oracle."""
+    """8M Gaussians at 7680x4320 (129 600 tiles, two partition passes of 9-bit digits, the blend
+    variant with fewer resident waves), 2 % of the splats enlarged: the whole frame against the oracle."""
     sc = config3_scene
     ref = _check_frame(oracle, sc, sc.cameras[0], 1 << 25)
     assert ref["K"] > 10_000_000
@@ -617,8 +617,8 @@ def test_sort_bits_above_the_range_stay_with_their_pair():
 
 
 def test_sort_more_tile_ids_than_the_segment_table():
-    """16400 x 16400 pixels = 1 050 625 tiles: 21 tile bits, three partition passes, and segment
-    bounds found by search instead of the table."""
+    """16400 x 16400 pixels = 1 050 625 tiles: 21 tile bits, three partition passes of 9-bit digits,
+    and segment bounds found by search instead of the table."""
     rng = np.random.default_rng(78)
     W = H = 16400
     n = 300_000
