@@ -673,39 +673,44 @@ __device__ __forceinline__ uint64_t from_lane_xor64(uint64_t x)
     return ((uint64_t)from_lane_xor<kJ>((uint32_t)(x >> 32)) << 32) | from_lane_xor<kJ>((uint32_t)x);
 }
 
-// The network over kT register slots of every lane, 64 * kT elements.  The merge width k runs
-// in a loop; the compare distances j are written out, so the code holds every exchange pattern
-// once whatever the number of stages.
+// The network over kT register slots of every lane, 64 * kT elements, element i in slot i % kT of
+// lane i / kT.  A compare distance below kT pairs two slots of one lane (registers only); a
+// larger one pairs the same slot of two lanes: 21 of the (log n)(log n + 1)/2 exchange steps
+// cross lanes whatever kT is, where the slot-major layout (element i in lane i % 64) makes it
+// 33 of 36 for 256 elements and 45 of 55 for 1024.  The merge width k runs in a loop; the compare
+// distances j are written out, so the code holds every exchange pattern once whatever the number
+// of stages.
 template <int kT>
 __device__ __forceinline__ void bitonic_network(uint64_t (&c)[kT], int lane)
 {
     constexpr int n = kT * kWave;
 #pragma unroll 1
     for (int k = 2; k <= n; k <<= 1) {
-        bool ascending[kT];                 // element t*64 + lane sits in an ascending run of width k
+        bool ascending[kT];                 // element lane*kT + t sits in an ascending run of width k
 #pragma unroll
-        for (int t = 0; t < kT; t++) ascending[t] = ((t * kWave + lane) & k) == 0;
+        for (int t = 0; t < kT; t++) ascending[t] = ((lane * kT + t) & k) == 0;
 #pragma unroll
         for (int j = n / 2; j > 0; j >>= 1) {
             if (j >= k) continue;
-            if (j >= kWave) {
-                const int jt = j / kWave;
+            if (j < kT) {
 #pragma unroll
                 for (int t = 0; t < kT; t++) {
-                    if ((t & jt) != 0) continue;
-                    const int t2 = t | jt;
+                    if ((t & j) != 0) continue;
+                    const int t2 = t | j;
                     const bool swap = (c[t] > c[t2]) == ascending[t];
                     const uint64_t a = swap ? c[t2] : c[t], b = swap ? c[t] : c[t2];
                     c[t] = a; c[t2] = b;
                 }
             } else {
-                const bool lower = (lane & j) == 0;
+                constexpr int kLanesMax = kWave / 2;
+                const int jl = j / kT;                                   // 1, 2, ... 32
+                const bool lower = (lane & jl) == 0;
 #pragma unroll
                 for (int t = 0; t < kT; t++) {
                     const uint64_t mine = c[t];
-                    const uint64_t other = j == 1 ? from_lane_xor64<1>(mine) : j == 2 ? from_lane_xor64<2>(mine)
-                                         : j == 4 ? from_lane_xor64<4>(mine) : j == 8 ? from_lane_xor64<8>(mine)
-                                         : j == 16 ? from_lane_xor64<16>(mine) : from_lane_xor64<32>(mine);
+                    const uint64_t other = jl == 1 ? from_lane_xor64<1>(mine) : jl == 2 ? from_lane_xor64<2>(mine)
+                                         : jl == 4 ? from_lane_xor64<4>(mine) : jl == 8 ? from_lane_xor64<8>(mine)
+                                         : jl == 16 ? from_lane_xor64<16>(mine) : from_lane_xor64<kLanesMax>(mine);
                     const bool keep_min = lower == ascending[t];
                     const bool take = (other < mine) == keep_min;       // the words are never equal
                     c[t] = take ? other : mine;
@@ -715,30 +720,25 @@ __device__ __forceinline__ void bitonic_network(uint64_t (&c)[kT], int lane)
     }
 }
 
-// bitonic_network over the first kUse of the kT slots
-template <int kUse, int kT>
-__device__ __forceinline__ void bitonic_network_of(uint64_t (&c)[kT], int lane)
+// Sorts the segment [lo, hi) of tile id v with the network over kUse slots per lane, 64 * kUse >= hi - lo.
+// Every word carries its element's position, so it does not matter which slot an element starts
+// in: the loads are the contiguous ones (element t*64 + lane in slot t), the network leaves rank
+// lane*kUse + t in slot t, and the sorted pairs go through LDS to be stored contiguously again.
+// s_v holds three arrays of kStride words: values by position, sorted depths, sorted values.
+template <int kUse, int kStride>
+__device__ __forceinline__ void sort_segment_bitonic_of(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
+                                                        uint32_t v, int lo, int hi, uint32_t* __restrict__ seg_flags,
+                                                        uint32_t* s_v)
 {
-    uint64_t h[kUse];
-#pragma unroll
-    for (int t = 0; t < kUse; t++) h[t] = c[t];
-    bitonic_network<kUse>(h, lane);
-#pragma unroll
-    for (int t = 0; t < kUse; t++) c[t] = h[t];
-}
-
-template <int kT>
-__device__ __forceinline__ void sort_segment_bitonic(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
-                                                     uint32_t v, int lo, int hi, uint32_t* __restrict__ seg_flags,
-                                                     uint32_t* s_v)
-{
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & (kWave - 1);
     const int len = hi - lo;
     const uint32_t upper = (uint32_t)(keys[lo] >> 32);
-    uint64_t c[kT];
+    uint32_t* const s_depth = s_v + kStride;
+    uint32_t* const s_value = s_v + 2 * kStride;
+    uint64_t c[kUse];
     bool mixed = false;
 #pragma unroll
-    for (int t = 0; t < kT; t++) {
+    for (int t = 0; t < kUse; t++) {
         const int i = t * kWave + lane;
         c[t] = ~0ull;
         if (i < len) {
@@ -752,22 +752,42 @@ __device__ __forceinline__ void sort_segment_bitonic(uint64_t* __restrict__ keys
         if (seg_flags && lane == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
         return;
     }
-    // the network over the smallest power of two of register slots that holds the segment
-    if (len <= kWave) bitonic_network_of<1>(c, lane);
-    else if (kT >= 2 && len <= 2 * kWave) bitonic_network_of<(kT >= 2 ? 2 : 1)>(c, lane);
-    else if (kT >= 4 && len <= 4 * kWave) bitonic_network_of<(kT >= 4 ? 4 : 1)>(c, lane);
-    else if (kT >= 8 && len <= 8 * kWave) bitonic_network_of<(kT >= 8 ? 8 : 1)>(c, lane);
-    else bitonic_network_of<kT>(c, lane);
+    bitonic_network<kUse>(c, lane);
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int t = 0; t < kT; t++) {
-        const int i = t * kWave + lane;
-        if (i < len) {
-            keys[lo + i] = ((uint64_t)upper << 32) | (c[t] >> 32);
-            values[lo + i] = s_v[(uint32_t)c[t]];
+    for (int t = 0; t < kUse; t++) {
+        const int r = lane * kUse + t;
+        if (r < len) {
+            s_depth[r] = (uint32_t)(c[t] >> 32);
+            s_value[r] = s_v[(uint32_t)c[t]];
         }
     }
     __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int t = 0; t < kUse; t++) {
+        const int i = t * kWave + lane;
+        if (i < len) {
+            keys[lo + i] = ((uint64_t)upper << 32) | s_depth[i];
+            values[lo + i] = s_value[i];
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+}
+
+// The network over the smallest power of two of register slots (at most kT) that holds the segment.
+// s_v: 3 * kT * 64 words.
+template <int kT>
+__device__ __forceinline__ void sort_segment_bitonic(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
+                                                     uint32_t v, int lo, int hi, uint32_t* __restrict__ seg_flags,
+                                                     uint32_t* s_v)
+{
+    constexpr int kS = kT * kWave;
+    const int len = hi - lo;
+    if (len <= kWave) sort_segment_bitonic_of<1, kS>(keys, values, v, lo, hi, seg_flags, s_v);
+    else if (kT >= 2 && len <= 2 * kWave) sort_segment_bitonic_of<(kT >= 2 ? 2 : 1), kS>(keys, values, v, lo, hi, seg_flags, s_v);
+    else if (kT >= 4 && len <= 4 * kWave) sort_segment_bitonic_of<(kT >= 4 ? 4 : 1), kS>(keys, values, v, lo, hi, seg_flags, s_v);
+    else if (kT >= 8 && len <= 8 * kWave) sort_segment_bitonic_of<(kT >= 8 ? 8 : 1), kS>(keys, values, v, lo, hi, seg_flags, s_v);
+    else sort_segment_bitonic_of<kT, kS>(keys, values, v, lo, hi, seg_flags, s_v);
 }
 
 // One wave per workgroup; with a table of segment starts the workgroup looks at kIds tile ids
@@ -782,7 +802,7 @@ __global__ __launch_bounds__(kWave) void segment_sort_wave_kernel(
     uint32_t* __restrict__ list2, uint32_t* __restrict__ list3,
     uint32_t list_cap0, uint32_t list_cap1, uint32_t list_cap2, uint32_t list_cap3)
 {
-    __shared__ uint32_t s_v[kT * kWave];
+    __shared__ uint32_t s_v[3 * kT * kWave];      // values by position, sorted depths, sorted values
     const int lane = threadIdx.x;
     if (!seg_start) {
         const uint32_t v = blockIdx.x;
@@ -826,7 +846,7 @@ __global__ __launch_bounds__(kWave) void segment_sort_wave_list_kernel(
     uint32_t* __restrict__ seg_flags, const uint32_t* __restrict__ list, const uint32_t* __restrict__ list_count,
     uint32_t list_cap)
 {
-    __shared__ uint32_t s_v[kT * kWave];
+    __shared__ uint32_t s_v[3 * kT * kWave];      // values by position, sorted depths, sorted values
     const uint32_t shard = blockIdx.x % kListShards;
     const uint32_t count = list_count[shard];
     for (uint32_t i = blockIdx.x / kListShards; i < count; i += gridDim.x / kListShards) {
