@@ -18,11 +18,13 @@
  *                         brute-force soundness over pixel centres             pinned
  *   key packing           integer identities, multiset invariants              pinned
  *   sh_color              scipy real spherical harmonics + 3DGS sign table     pinned
- *   stale rows            sentinel test                                        pinned
+ *   stale rows            sentinel test; one-tile rectangle without a key      pinned
  *   sort                  numpy stable argsort                                 pinned
  *   ranges                numpy searchsorted                                   pinned
  *   render                closed form 1 and 2 Gaussians, float64 per-pixel
  *                         brute force on small scenes, early-out bound         pinned
+ *   preprocess -> render  rotated anisotropic Gaussian: op exp(-d^T S^-1 d/2)
+ *                         with S inverted in float64 (the conic's cross term)  pinned
  *   cov3d                 float64 R S S R^T                                    pinned
  * Not pinnable by anything available offline: the bit patterns of the PTX
  * .approx instructions the reference executes, nvcc's FMA contraction choices
