@@ -5,6 +5,9 @@
 #include <stdint.h>
 #include <stddef.h>
 
+#include <thread>
+#include <tuple>
+
 #include "../../include/flashgs_hip.h"
 
 namespace fgs {
@@ -31,6 +34,14 @@ inline int bit_length(uint32_t n)
     int b = 0;
     while (n) { b++; n >>= 1; }
     return b;
+}
+
+// What the library's per-stream memory is keyed by.  hipStreamPerThread is one handle that names a
+// different stream in every host thread, so there the thread is part of the key.
+typedef std::tuple<int, hipStream_t, std::thread::id> StreamKey;
+inline StreamKey stream_key(int device, hipStream_t stream)
+{
+    return StreamKey(device, stream, stream == hipStreamPerThread ? std::this_thread::get_id() : std::thread::id());
 }
 
 constexpr int kWave = 64;

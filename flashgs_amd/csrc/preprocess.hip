@@ -942,7 +942,7 @@ struct Scratch {
 };
 
 constexpr int kMaxDevices = 64;
-std::map<std::pair<int, hipStream_t>, Scratch> g_scratch;
+std::map<StreamKey, Scratch> g_scratch;
 std::mutex g_mutex;
 std::atomic<unsigned> g_spin_limit{kSpinLimit};
 
@@ -951,7 +951,7 @@ std::atomic<unsigned> g_spin_limit{kSpinLimit};
 int acquire_scratch(int device, int num_blocks, hipStream_t stream, Scratch** out)
 {
     *out = nullptr;
-    Scratch& s = g_scratch[std::make_pair(device, stream)];
+    Scratch& s = g_scratch[stream_key(device, stream)];
     if (s.capacity < (size_t)num_blocks) {
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         if (stream) FGS_HIP_TRY(hipStreamIsCapturing(stream, &capture));

@@ -41,7 +41,7 @@ constexpr int kOrderBins = 128;            // everything from 2032 entries up sh
 // stream that is being captured and has no table yet cannot allocate one and uses this
 // per-device table instead, which captured blends on one device then share.
 __device__ uint32_t g_tile_order[kOrderCap];
-std::map<std::pair<int, hipStream_t>, uint32_t*> g_order_tables;
+std::map<StreamKey, uint32_t*> g_order_tables;
 std::mutex g_order_mutex;
 
 int tile_order_table(hipStream_t stream, uint32_t** out)
@@ -49,7 +49,7 @@ int tile_order_table(hipStream_t stream, uint32_t** out)
     int device = 0;
     FGS_HIP_TRY(hipGetDevice(&device));
     std::lock_guard<std::mutex> lock(g_order_mutex);
-    uint32_t*& table = g_order_tables[std::make_pair(device, stream)];
+    uint32_t*& table = g_order_tables[stream_key(device, stream)];
     if (!table) {
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         if (stream) FGS_HIP_TRY(hipStreamIsCapturing(stream, &capture));
