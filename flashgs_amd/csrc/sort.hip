@@ -207,34 +207,8 @@ __global__ __launch_bounds__(kOffsetThreads) void offsets_kernel(uint32_t* __res
     }
 }
 
-// The same for a short list (at most kSmallRows histogram rows): one workgroup, one thread per
-// digit, no chunk sums in between.
+// A list of at most kSmallRows histogram rows needs neither: the scatter workgroups add the rows up themselves.
 constexpr int kSmallRows = 64;
-
-template <class Shape>
-__global__ __launch_bounds__(Shape::kBinsP) void offsets_small_kernel(uint32_t* __restrict__ hist, int tiles)
-{
-    constexpr int kB = Shape::kBinsP;
-    __shared__ uint32_t s_wave[kB / kWave];
-    const int d = threadIdx.x;
-    const int lane = d & (kWave - 1), wave = d / kWave;
-    uint32_t c[kSmallRows];
-#pragma unroll
-    for (int t = 0; t < kSmallRows; t++) c[t] = t < tiles ? hist[(size_t)t * kB + d] : 0u;
-    uint32_t total = 0;
-#pragma unroll
-    for (int t = 0; t < kSmallRows; t++) total += c[t];
-    uint32_t incl = wave_inclusive_sum(total);
-    if (lane == kWave - 1) s_wave[wave] = incl;
-    __syncthreads();
-    uint32_t run = incl - total;
-    for (int w = 0; w < wave; w++) run += s_wave[w];
-#pragma unroll
-    for (int t = 0; t < kSmallRows; t++) {
-        if (t < tiles) hist[(size_t)t * kB + d] = run;
-        run += c[t];
-    }
-}
 
 // ---- step 3: stable scatter ---------------------------------------------------------------------------
 
@@ -243,7 +217,8 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
     const uint64_t* __restrict__ keys_in, const uint32_t* __restrict__ values_in,
     uint64_t* __restrict__ keys_out, uint32_t* __restrict__ values_out,
     int n, int shift, int nbits,
-    const uint32_t* __restrict__ start)          // [blocks][bins] from offsets_kernel
+    const uint32_t* __restrict__ start,          // [blocks][bins] from offsets_kernel, or ...
+    int raw_rows)                                // ... if > 0, the raw_rows histogram rows themselves (a short list)
 {
     constexpr int kB = Shape::kBinsP, kItems = Shape::kItems, kTile = Shape::kTile, kPer = Shape::kPerThread;
     // per-wave digit counts, then per-wave digit offsets: at most kTile, so 16 bits do, and with
@@ -279,8 +254,37 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
         val[i] = off < in_tile ? values_in[tile_base + off] : 0u;
     }
     uint32_t my_start[kPer];
+    if (raw_rows == 0) {
 #pragma unroll
-    for (int q = 0; q < kPer; q++) my_start[q] = start[(size_t)tile * kB + q * kSortBlock + tid];
+        for (int q = 0; q < kPer; q++) my_start[q] = start[(size_t)tile * kB + q * kSortBlock + tid];
+    } else {
+        // A list of at most kSmallRows blocks: every workgroup adds up the histogram rows itself
+        // (the digit totals, and what the blocks in front of it hold of each digit), which
+        // saves the launch that would do it.
+        uint32_t total[kPer], before[kPer], incl[kPer];
+#pragma unroll
+        for (int q = 0; q < kPer; q++) {
+            const int d = q * kSortBlock + tid;
+            total[q] = 0; before[q] = 0;
+#pragma unroll 8
+            for (int b = 0; b < raw_rows; b++) {
+                const uint32_t c = start[(size_t)b * kB + d];
+                total[q] += c;
+                before[q] += b < tile ? c : 0u;
+            }
+            incl[q] = wave_inclusive_sum(total[q]);
+            if (lane == kWave - 1) s_wave_sum[q * kSortWaves + wave] = incl[q];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < kPer; q++) {
+            uint32_t digit_base = incl[q] - total[q];
+#pragma unroll
+            for (int w = 0; w < kPer * kSortWaves; w++)
+                if (w < q * kSortWaves + wave) digit_base += s_wave_sum[w];
+            my_start[q] = digit_base + before[q];
+        }
+    }
 #pragma unroll
     for (int w = 0; w < kSortWaves; w++)
 #pragma unroll
@@ -1021,15 +1025,13 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
             const int shift = 32 + Shape::kBits * p;
             const int nbits = tile_bits - Shape::kBits * p < Shape::kBits ? tile_bits - Shape::kBits * p : Shape::kBits;
             hipLaunchKernelGGL((count_kernel<Shape>), dim3(g.tiles), dim3(kSortBlock), 0, st, src_k, n, shift, nbits, hist);
-            if (g.tiles <= kSmallRows) {
-                hipLaunchKernelGGL((offsets_small_kernel<Shape>), dim3(1), dim3(Shape::kBinsP), 0, st, hist, g.tiles);
-            } else {
+            if (g.tiles > kSmallRows) {
                 hipLaunchKernelGGL((chunk_sum_kernel<Shape>), dim3(g.chunks), dim3(Shape::kBinsP), 0, st, hist, g.tiles, g.chunk, chunk_sums);
                 hipLaunchKernelGGL((offsets_kernel<Shape>), dim3(g.chunks), dim3(g.chunks > 16 ? kOffsetThreads : Shape::kBinsP), 0, st,
                                    hist, g.tiles, g.chunk, chunk_sums, g.chunks);
             }
             hipLaunchKernelGGL((scatter_kernel<Shape>), dim3(g.tiles), dim3(kSortBlock), 0, st,
-                               src_k, src_v, dst_k, dst_v, n, shift, nbits, hist);
+                               src_k, src_v, dst_k, dst_v, n, shift, nbits, hist, g.tiles <= kSmallRows ? g.tiles : 0);
             src_k = dst_k;
             src_v = dst_v;
         }
