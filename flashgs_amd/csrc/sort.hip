@@ -114,11 +114,18 @@ __device__ __forceinline__ uint32_t digit_of(uint64_t key, int shift, uint32_t m
 
 template <class Shape>
 __global__ __launch_bounds__(kSortBlock) void count_kernel(const uint64_t* __restrict__ keys, int n,
-                                                           int shift, int nbits, uint32_t* __restrict__ hist)
+                                                           int shift, int nbits, uint32_t* __restrict__ hist,
+                                                           uint32_t* __restrict__ seg_flags, uint32_t flag_words,
+                                                           uint32_t* __restrict__ seg_counts)
 {
     constexpr int kB = Shape::kBinsP;
     __shared__ uint32_t h[kB];
     const int tid = threadIdx.x;
+    if (seg_flags) {        // the last pass also clears what the segment launches append to
+        const uint32_t gid = blockIdx.x * kSortBlock + tid;
+        for (uint32_t w = gid; w < flag_words; w += gridDim.x * kSortBlock) seg_flags[w] = 0;
+        if (gid < (uint32_t)(kListClasses * kListShards)) seg_counts[gid] = 0;
+    }
 #pragma unroll
     for (int q = 0; q < Shape::kPerThread; q++) h[q * kSortBlock + tid] = 0;
     __syncthreads();
@@ -212,13 +219,22 @@ constexpr int kSmallRows = 64;
 
 // ---- step 3: stable scatter ---------------------------------------------------------------------------
 
-template <class Shape>
+// With kTable (the last pass of at most two) the launch also writes the table of segment starts,
+// seg_start[v] = first index of the output whose tile field is >= v, v in [0, ids], ids = 2^(bits of
+// the tile field).  The input of that pass is ordered by the low part of the tile field (the bits
+// below this pass's digit), so the first pair with low part >= L lies in exactly one workgroup's
+// block, and that workgroup writes the entries (d, L) of every digit d: the destination of its
+// first pair with digit d and low part >= L, or, if it has none, the end of its run of digit d,
+// which is where the next workgroup's run of d begins.  Every entry has one writer, empty ids
+// included, and no launch has to read the keys again.
+template <class Shape, bool kTable>
 __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
     const uint64_t* __restrict__ keys_in, const uint32_t* __restrict__ values_in,
     uint64_t* __restrict__ keys_out, uint32_t* __restrict__ values_out,
     int n, int shift, int nbits,
     const uint32_t* __restrict__ start,          // [blocks][bins] from offsets_kernel, or ...
-    int raw_rows)                                // ... if > 0, the raw_rows histogram rows themselves (a short list)
+    int raw_rows,                                // ... if > 0, the raw_rows histogram rows themselves (a short list)
+    int* __restrict__ seg_start)                 // kTable: [2^(shift - 32 + nbits) + 1]
 {
     constexpr int kB = Shape::kBinsP, kItems = Shape::kItems, kTile = Shape::kTile, kPer = Shape::kPerThread;
     // per-wave digit counts, then per-wave digit offsets: at most kTile, so 16 bits do, and with
@@ -360,16 +376,51 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
     }
     __syncthreads();
 
+    // The low parts L whose first pair (the first of the input with low part >= L) lies in this
+    // block: those above the low part of the pair in front of the block, up to that of the
+    // block's last pair; the last block also takes the ones no pair reaches.
+    const int low_bits = shift - 32;
+    const uint32_t low_mask = (1u << low_bits) - 1u;
+    int own_lo = 0, own_hi = -1;
+    if (kTable) {
+        if (tile > 0) own_lo = (int)((uint32_t)(keys_in[tile_base - 1] >> 32) & low_mask) + 1;
+        own_hi = tile == (int)gridDim.x - 1 ? (int)low_mask
+                                            : (int)((uint32_t)(keys_in[tile_base + in_tile - 1] >> 32) & low_mask);
+    }
+
     // write out: neighbouring threads hold neighbouring ranked slots
 #pragma unroll
     for (int i = 0; i < kItems; i++) {
         const int p = i * kSortBlock + tid;
         if (p < in_tile) {
             const uint64_t k = s_keys[p];
-            const uint32_t dst = s_global[digit_of(k, shift, mask)] + (uint32_t)p;
+            const uint32_t d = digit_of(k, shift, mask);
+            const uint32_t dst = s_global[d] + (uint32_t)p;
             keys_out[dst] = k;
             values_out[dst] = s_values[p];
+            if (kTable && own_lo <= own_hi) {
+                // the first pair of digit d with a low part >= L, for every owned L up to its own
+                const int low = (int)((uint32_t)(k >> 32) & low_mask);
+                int prev = own_lo - 1;
+                if (p > (int)s_bin_start[d]) prev = (int)((uint32_t)(s_keys[p - 1] >> 32) & low_mask);
+                for (int l = max(prev + 1, own_lo); l <= low; l++) seg_start[(d << low_bits) | (uint32_t)l] = (int)dst;
+            }
         }
+    }
+    if (kTable) {
+        if (own_lo <= own_hi) {
+            // owned low parts above the last pair of a digit's run: the end of the run
+#pragma unroll
+            for (int q = 0; q < kPer; q++) {
+                const uint32_t d = (uint32_t)(q * kSortBlock + tid);
+                if (d > mask) continue;
+                int last = own_lo - 1;
+                if (total[q]) last = (int)((uint32_t)(s_keys[(uint32_t)s_bin_start[d] + total[q] - 1u] >> 32) & low_mask);
+                const int end = (int)(my_start[q] + total[q]);
+                for (int l = max(last + 1, own_lo); l <= own_hi; l++) seg_start[(d << low_bits) | (uint32_t)l] = end;
+            }
+        }
+        if (tile == 0 && tid == 0) seg_start[(size_t)1 << (low_bits + nbits)] = n;
     }
 }
 
@@ -959,7 +1010,7 @@ __global__ __launch_bounds__(kSortBlock) void segment_sort_general_kernel(
 }
 
 constexpr int kCapTiny = 512, kCapSmall = 1024, kCapMedium = 4096, kCapLarge = 8192;
-constexpr uint32_t kOneLaunchIds = 16384;    // up to this many tile ids one launch sorts every segment of up to kCapSmall pairs
+constexpr uint32_t kOneLaunchIds = 32768;    // up to this many tile ids one launch sorts every segment of up to kCapSmall pairs
 
 
 } // namespace
@@ -1011,11 +1062,26 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
     uint32_t* hist = (uint32_t*)(list_sorting_space + ws.hist);
     uint32_t* chunk_sums = (uint32_t*)(list_sorting_space + ws.chunk_sums);
 
+    // The table of segment starts (with it the flag words and the lists of the longer segments)
+    // exists up to kMaxTableIds tile ids.  The last partition pass writes it when there are at
+    // most two passes: with more, one workgroup could own 2^18 and more entries of a sparse frame.
+    const uint32_t ids = 1u << tile_bits;
+    int* seg_start = nullptr;
+    uint32_t* seg_flags = nullptr;
+    uint32_t* seg_counts = nullptr;
+    if (n > 1 && ids <= kMaxTableIds) {
+        seg_start = (int*)(list_sorting_space + ws.seg_start);
+        seg_flags = (uint32_t*)(list_sorting_space + ws.seg_flags);
+        seg_counts = (uint32_t*)(list_sorting_space + ws.seg_lists);
+    }
+    bool table_by_scatter = false;
+
     // 1. stable partition by tile id, least significant tile digit first
     auto partition = [&](auto shape) {
         using Shape = decltype(shape);
         const PassGrid g = pass_grid(n, Shape::kTile);
         const int passes = (tile_bits + Shape::kBits - 1) / Shape::kBits;
+        table_by_scatter = seg_start && passes <= 2;
         const uint64_t* src_k = gaussian_keys_unsorted;
         const uint32_t* src_v = gaussian_values_unsorted;
         for (int p = 0; p < passes; p++) {
@@ -1024,14 +1090,20 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
             uint32_t* dst_v = to_sorted ? gaussian_values_sorted : alt_values;
             const int shift = 32 + Shape::kBits * p;
             const int nbits = tile_bits - Shape::kBits * p < Shape::kBits ? tile_bits - Shape::kBits * p : Shape::kBits;
-            hipLaunchKernelGGL((count_kernel<Shape>), dim3(g.tiles), dim3(kSortBlock), 0, st, src_k, n, shift, nbits, hist);
+            const bool last = p == passes - 1;
+            hipLaunchKernelGGL((count_kernel<Shape>), dim3(g.tiles), dim3(kSortBlock), 0, st, src_k, n, shift, nbits, hist,
+                               last ? seg_flags : nullptr, (ids + 31) / 32, seg_counts);
             if (g.tiles > kSmallRows) {
                 hipLaunchKernelGGL((chunk_sum_kernel<Shape>), dim3(g.chunks), dim3(Shape::kBinsP), 0, st, hist, g.tiles, g.chunk, chunk_sums);
                 hipLaunchKernelGGL((offsets_kernel<Shape>), dim3(g.chunks), dim3(g.chunks > 16 ? kOffsetThreads : Shape::kBinsP), 0, st,
                                    hist, g.tiles, g.chunk, chunk_sums, g.chunks);
             }
-            hipLaunchKernelGGL((scatter_kernel<Shape>), dim3(g.tiles), dim3(kSortBlock), 0, st,
-                               src_k, src_v, dst_k, dst_v, n, shift, nbits, hist, g.tiles <= kSmallRows ? g.tiles : 0);
+            if (last && table_by_scatter)
+                hipLaunchKernelGGL((scatter_kernel<Shape, true>), dim3(g.tiles), dim3(kSortBlock), 0, st,
+                                   src_k, src_v, dst_k, dst_v, n, shift, nbits, hist, g.tiles <= kSmallRows ? g.tiles : 0, seg_start);
+            else
+                hipLaunchKernelGGL((scatter_kernel<Shape, false>), dim3(g.tiles), dim3(kSortBlock), 0, st,
+                                   src_k, src_v, dst_k, dst_v, n, shift, nbits, hist, g.tiles <= kSmallRows ? g.tiles : 0, (int*)nullptr);
             src_k = dst_k;
             src_v = dst_v;
         }
@@ -1041,20 +1113,14 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
 
     // 2. every tile id's segment by depth, in place in the sorted buffers
     if (n > 1) {
-        const uint32_t ids = 1u << tile_bits;
-        int* seg_start = nullptr;
-        uint32_t* seg_flags = nullptr;
-        if (ids <= kMaxTableIds) {
-            seg_start = (int*)(list_sorting_space + ws.seg_start);
-            seg_flags = (uint32_t*)(list_sorting_space + ws.seg_flags);
+        if (seg_start && !table_by_scatter) {
             const unsigned blocks = (unsigned)(((size_t)n + 256 * kStartsPerThread - 1) / (256 * kStartsPerThread));
             hipLaunchKernelGGL(segment_starts_kernel, dim3(blocks), dim3(256), 0, st,
-                               (const uint64_t*)gaussian_keys_sorted, n, tile_mask, ids, seg_start, seg_flags,
-                               (uint32_t*)(list_sorting_space + ws.seg_lists));
+                               (const uint64_t*)gaussian_keys_sorted, n, tile_mask, ids, seg_start, seg_flags, seg_counts);
         }
         uint64_t* ks = gaussian_keys_sorted;
         uint32_t* vs = gaussian_values_sorted;
-        uint32_t* seg_counts = (uint32_t*)(list_sorting_space + ws.seg_lists);
+        seg_counts = (uint32_t*)(list_sorting_space + ws.seg_lists);
         const uint32_t cap_small = (uint32_t)(n / 512 + 2), cap_medium = (uint32_t)(n / 1024 + 2), cap_large = (uint32_t)(n / 4096 + 2),
                        cap_long = (uint32_t)(n / 8192 + 2);
         uint32_t* list_small = seg_counts + 128;
@@ -1076,8 +1142,8 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         // of the launch).  With a table the launch also lists the longer segments.
         // A frame of few tiles has few segments of 513..1024 pairs, about one wave per SIMD, and a
         // launch of their own lasts as long as one such sort: there the first launch takes them
-        // too, with 16 register slots (1080p: -15 us; at 4K no difference, at 8K +65 us, because
-        // the launch over 131 072 ids then runs at 3 instead of 7 waves per SIMD).
+        // too, with 16 register slots (1080p: -15 us, 4K: -8 us; at 8K +40 us, because the launch
+        // over 131 072 ids, most of them under 128 pairs, then runs at fewer waves per SIMD).
         const bool one_wave_launch = seg_start && ids <= kOneLaunchIds;
         if (one_wave_launch)
             hipLaunchKernelGGL((segment_sort_wave_kernel<kCapSmall / kWave, 1>), dim3(ids), dim3(kWave),

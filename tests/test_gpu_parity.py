@@ -616,6 +616,37 @@ def test_sort_bits_above_the_range_stay_with_their_pair():
     _sort_case(tile, depth, W, H, junk=junk, seed=1)
 
 
+@pytest.mark.parametrize("W,H,n", [(16, 16, 5000), (256, 16, 9000), (160, 128, 70_000), (3840, 2160, 300),
+                                   (7680, 4320, 40), (8208, 8208, 200_000), (8208, 8208, 90)])
+def test_sort_segment_table_shapes(W, H, n):
+    """The table of segment starts under every way it is produced: one partition pass (up to 256 tile
+    ids, one of them a frame of a single tile), two passes on a sparse frame (one workgroup owns every
+    entry, most tile ids empty, first and last tile in use), and 263 169 tiles (19 tile bits, three
+    passes, where a launch of its own reads the sorted keys)."""
+    rng = np.random.default_rng(W + n)
+    tiles = ((W + 15) // 16) * ((H + 15) // 16)
+    tile = rng.integers(0, tiles, n).astype(np.uint32)
+    tile[:3] = tiles - 1
+    tile[3:5] = 0
+    depth = rng.uniform(0.2, 90.0, n).astype(np.float32)
+    depth[::4] = np.float32(2.5)
+    _sort_case(tile, depth.view(np.uint32), W, H, seed=n)
+
+
+def test_sort_low_digit_changes_at_block_boundaries():
+    """Second partition pass whose input blocks (4096 pairs) end exactly where the low tile digit
+    changes, with low digits that no pair has in between: every entry of the segment table still
+    has exactly one writer."""
+    rng = np.random.default_rng(4096)
+    W, H = 3840, 2160
+    lows = np.array([3, 7, 7, 200, 201, 255], np.uint32)
+    high = rng.integers(0, 126, (lows.size, 4096)).astype(np.uint32)
+    tile = (high * 256 + lows[:, None]).reshape(-1)
+    tile = tile[rng.permutation(tile.size)]
+    depth = rng.integers(0, 1 << 32, tile.size, dtype=np.uint64).astype(np.uint32)
+    _sort_case(tile, depth, W, H, seed=3)
+
+
 def test_sort_more_tile_ids_than_the_segment_table():
     """16400 x 16400 pixels = 1 050 625 tiles: 21 tile bits, three partition passes of 9-bit digits,
     and segment bounds found by search instead of the table."""
