@@ -8,14 +8,16 @@
 //
 //  1. Partition by tile id: one stable counting pass per 8 bits of tile id (two passes for up to
 //     65536 tiles; above that digits of 9 bits, so an 8K frame of 129 600 tiles still takes two).
-//     A pass is count -> offsets -> scatter: `count_kernel` builds one digit
-//     histogram per block of 4096 pairs (3840 with 9-bit digits), `chunk_sum_kernel` + `offsets_kernel` turn the
-//     histograms into the exclusive start of every (block, digit) run, and `scatter_kernel` ranks
-//     its block in LDS (wave64 ballot matching, so equal digits keep their input order) and
-//     writes each run to its start.  No workgroup ever waits for another one.
-//  2. Sort every tile's segment by the 32 depth bits without touching memory in between:
-//     `segment_starts_kernel` tabulates where each tile id's segment begins, then segments are
-//     handled by size class.  Up to 1024 pairs one wave holds the segment in registers as 64-bit
+//     A pass is count -> offsets -> scatter: `count_chunk_kernel` builds one digit histogram per
+//     block of 4096 pairs (3840 with 9-bit digits) and the sums of every chunk of blocks,
+//     `offsets_kernel` turns them into the exclusive start of every (block, digit) run, and
+//     `scatter_kernel` ranks its block in LDS (wave64 ballot matching, so equal digits keep
+//     their input order) and writes each run to its start.  A list of up to 64 blocks takes
+//     count -> scatter.  No workgroup ever waits for another one.
+//  2. Sort every tile's segment by the 32 depth bits without touching memory in between: the
+//     last scatter pass also tabulates where each tile id's segment begins (with more than two
+//     passes `segment_starts_kernel` does, from the sorted keys), then segments are handled by
+//     size class.  Up to 1024 pairs one wave holds the segment in registers as 64-bit
 //     words depth << 32 | position and runs a bitonic network on them (all words differ, so the
 //     result is that of a stable sort by depth); lane exchanges inside a row of 16 lanes are
 //     data-parallel-primitive moves.  Up to 4096 (8 waves) and 8192 pairs (16 waves) a workgroup
@@ -33,7 +35,6 @@ namespace {
 constexpr int kBins = 256;                      // counters of a counting pass inside a segment (8-bit digits)
 constexpr int kSortBlock = 256;
 constexpr int kSortWaves = kSortBlock / kWave;
-constexpr int kMinChunk = 16;                   // fewest histogram rows summed by one chunk_sum workgroup
 
 // Shape of a partition pass: digits of kBitsT bits, kItemsT pairs per thread.  Up to 65 536 tiles
 // two passes of 8 bits do; above that (an 8K frame has 129 600) digits of 9 bits keep it at two
@@ -77,7 +78,7 @@ PassGrid pass_grid(int n, int tile)
 {
     PassGrid g;
     g.tiles = (n + tile - 1) / tile;
-    g.chunk = (g.tiles + 255) / 256 > kMinChunk ? (g.tiles + 255) / 256 : kMinChunk;     // at most ~256 chunks
+    g.chunk = g.tiles > 256 ? (g.tiles + 255) / 256 : 1;     // at most 256 chunks, one count workgroup each: about one per CU
     g.chunks = (g.tiles + g.chunk - 1) / g.chunk;
     return g;
 }
@@ -142,20 +143,74 @@ __global__ __launch_bounds__(kSortBlock) void count_kernel(const uint64_t* __res
         hist[(size_t)blockIdx.x * kB + q * kSortBlock + tid] = h[q * kSortBlock + tid];
 }
 
-// ---- step 2: exclusive start of every (block, digit) run ----------------------------------------
-// start[b][d] = sum of hist[*][d' < d] + sum of hist[b' < b][d]   (digit-major, then block)
+// The same for a list of more than kSmallRows blocks: one workgroup counts a whole chunk of
+// `chunk` consecutive blocks, blockDim.x / kSortBlock of them at a time, and so also has the
+// chunk's digit sums, which the offsets launch needs (a launch of their own would read the rows
+// back just to add them up).
+constexpr int kCountGroups = 4;
 
 template <class Shape>
-__global__ __launch_bounds__(Shape::kBinsP) void chunk_sum_kernel(const uint32_t* __restrict__ hist, int tiles, int chunk,
-                                                                  uint32_t* __restrict__ chunk_sums)
+__global__ __launch_bounds__(kCountGroups * kSortBlock) void count_chunk_kernel(
+    const uint64_t* __restrict__ keys, int n, int shift, int nbits, uint32_t* __restrict__ hist,
+    int tiles, int chunk, uint32_t* __restrict__ chunk_sums,
+    uint32_t* __restrict__ seg_flags, uint32_t flag_words, uint32_t* __restrict__ seg_counts)
 {
-    constexpr int kB = Shape::kBinsP;
-    const int d = threadIdx.x;
+    constexpr int kB = Shape::kBinsP, kPer = Shape::kPerThread;
+    __shared__ uint32_t h[kCountGroups][kB];
+    const int tid = threadIdx.x % kSortBlock, group = threadIdx.x / kSortBlock;
+    const int groups = (int)blockDim.x / kSortBlock;
+    if (seg_flags) {        // the last pass also clears what the segment launches append to
+        const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
+        for (uint32_t w = gid; w < flag_words; w += gridDim.x * blockDim.x) seg_flags[w] = 0;
+        if (gid < (uint32_t)(kListClasses * kListShards)) seg_counts[gid] = 0;
+    }
+    const uint32_t mask = (1u << nbits) - 1u;
     const int t0 = blockIdx.x * chunk, t1 = min(tiles, t0 + chunk);
-    uint32_t s = 0;
-    for (int t = t0; t < t1; t++) s += hist[(size_t)t * kB + d];
-    chunk_sums[(size_t)blockIdx.x * kB + d] = s;
+    uint32_t sum[kPer];
+#pragma unroll
+    for (int q = 0; q < kPer; q++) { sum[q] = 0; h[group][q * kSortBlock + tid] = 0; }
+    __syncthreads();
+    for (int first = t0; first < t1; first += groups) {      // the same trips for every group
+        const int row = first + group;
+        if (row < t1) {
+            const int base = row * Shape::kTile;
+            uint64_t k[Shape::kItems];
+#pragma unroll
+            for (int i = 0; i < Shape::kItems; i++) {
+                const int idx = base + i * kSortBlock + tid;
+                k[i] = idx < n ? keys[idx] : 0ull;
+            }
+#pragma unroll
+            for (int i = 0; i < Shape::kItems; i++)
+                if (base + i * kSortBlock + tid < n) atomicAdd(&h[group][digit_of(k[i], shift, mask)], 1u);
+        }
+        __syncthreads();
+        if (row < t1) {
+#pragma unroll
+            for (int q = 0; q < kPer; q++) {
+                const uint32_t c = h[group][q * kSortBlock + tid];
+                h[group][q * kSortBlock + tid] = 0;          // read and cleared by the same thread
+                hist[(size_t)row * kB + q * kSortBlock + tid] = c;
+                sum[q] += c;
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int q = 0; q < kPer; q++) h[group][q * kSortBlock + tid] = sum[q];
+    __syncthreads();
+    if (group == 0) {
+#pragma unroll
+        for (int q = 0; q < kPer; q++) {
+            uint32_t total = 0;
+            for (int g = 0; g < groups; g++) total += h[g][q * kSortBlock + tid];
+            chunk_sums[(size_t)blockIdx.x * kB + q * kSortBlock + tid] = total;
+        }
+    }
 }
+
+// ---- step 2: exclusive start of every (block, digit) run ----------------------------------------
+// start[b][d] = sum of hist[*][d' < d] + sum of hist[b' < b][d]   (digit-major, then block)
 
 // One workgroup per chunk, up to 1024 / bins threads per digit (blockDim.x / bins of them): the
 // chunk sums are few and the loop over them is latency-bound, so each group of `bins` threads
@@ -1091,10 +1146,14 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
             const int shift = 32 + Shape::kBits * p;
             const int nbits = tile_bits - Shape::kBits * p < Shape::kBits ? tile_bits - Shape::kBits * p : Shape::kBits;
             const bool last = p == passes - 1;
-            hipLaunchKernelGGL((count_kernel<Shape>), dim3(g.tiles), dim3(kSortBlock), 0, st, src_k, n, shift, nbits, hist,
-                               last ? seg_flags : nullptr, (ids + 31) / 32, seg_counts);
-            if (g.tiles > kSmallRows) {
-                hipLaunchKernelGGL((chunk_sum_kernel<Shape>), dim3(g.chunks), dim3(Shape::kBinsP), 0, st, hist, g.tiles, g.chunk, chunk_sums);
+            if (g.tiles <= kSmallRows) {
+                hipLaunchKernelGGL((count_kernel<Shape>), dim3(g.tiles), dim3(kSortBlock), 0, st, src_k, n, shift, nbits, hist,
+                                   last ? seg_flags : nullptr, (ids + 31) / 32, seg_counts);
+            } else {
+                const int groups = g.chunk < kCountGroups ? g.chunk : kCountGroups;
+                hipLaunchKernelGGL((count_chunk_kernel<Shape>), dim3(g.chunks), dim3(groups * kSortBlock), 0, st,
+                                   src_k, n, shift, nbits, hist, g.tiles, g.chunk, chunk_sums,
+                                   last ? seg_flags : nullptr, (ids + 31) / 32, seg_counts);
                 hipLaunchKernelGGL((offsets_kernel<Shape>), dim3(g.chunks), dim3(g.chunks > 16 ? kOffsetThreads : Shape::kBinsP), 0, st,
                                    hist, g.tiles, g.chunk, chunk_sums, g.chunks);
             }
