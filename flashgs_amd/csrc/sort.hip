@@ -309,6 +309,15 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
     const int tile_base = tile * kTile;
     const int in_tile = min(kTile, n - tile_base);
 
+    // The low parts L whose first pair (the first of the input with low part >= L) lies in this
+    // block: those above the low part of the pair in front of the block, up to that of the
+    // block's last pair; the last block also takes the ones no pair reaches.
+    const int low_bits = shift - 32;
+    const uint32_t low_mask = (1u << low_bits) - 1u;
+    __shared__ int s_own[2];
+    uint64_t edge_key = 0;          // thread 0: the pair in front of the block, thread 1: the block's last pair
+    if (kTable && tid < 2 && (tid == 1 || tile > 0)) edge_key = keys_in[tid == 0 ? tile_base - 1 : tile_base + in_tile - 1];
+
     // wave w owns slots [w*64*kItems, (w+1)*64*kItems) of the block, item-major; everything is
     // requested before the first use so the latencies overlap
     uint64_t key[kItems];
@@ -360,6 +369,10 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
     for (int w = 0; w < kSortWaves; w++)
 #pragma unroll
         for (int q = 0; q < kPer; q++) s_count[w][q * kSortBlock + tid] = 0;
+    if (kTable && tid < 2) {
+        const int low = (int)((uint32_t)(edge_key >> 32) & low_mask);
+        s_own[tid] = tid == 0 ? (tile > 0 ? low + 1 : 0) : (tile == (int)gridDim.x - 1 ? (int)low_mask : low);
+    }
     __syncthreads();
 
     // rank inside the wave: lanes with equal digits find each other with one ballot per digit bit
@@ -431,39 +444,46 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
     }
     __syncthreads();
 
-    // The low parts L whose first pair (the first of the input with low part >= L) lies in this
-    // block: those above the low part of the pair in front of the block, up to that of the
-    // block's last pair; the last block also takes the ones no pair reaches.
-    const int low_bits = shift - 32;
-    const uint32_t low_mask = (1u << low_bits) - 1u;
-    int own_lo = 0, own_hi = -1;
-    if (kTable) {
-        if (tile > 0) own_lo = (int)((uint32_t)(keys_in[tile_base - 1] >> 32) & low_mask) + 1;
-        own_hi = tile == (int)gridDim.x - 1 ? (int)low_mask
-                                            : (int)((uint32_t)(keys_in[tile_base + in_tile - 1] >> 32) & low_mask);
-    }
+    const int own_lo = kTable ? s_own[0] : 0, own_hi = kTable ? s_own[1] : -1;
 
-    // write out: neighbouring threads hold neighbouring ranked slots
+    // write out: neighbouring threads hold neighbouring ranked slots.  All LDS reads first (a slot
+    // past the end reads the last pair and stores nothing), so their latencies overlap.
+    {
+        uint64_t out_key[kItems];
+        uint32_t out_value[kItems], out_at[kItems];
 #pragma unroll
-    for (int i = 0; i < kItems; i++) {
-        const int p = i * kSortBlock + tid;
-        if (p < in_tile) {
-            const uint64_t k = s_keys[p];
-            const uint32_t d = digit_of(k, shift, mask);
-            const uint32_t dst = s_global[d] + (uint32_t)p;
-            keys_out[dst] = k;
-            values_out[dst] = s_values[p];
-            if (kTable && own_lo <= own_hi) {
-                // the first pair of digit d with a low part >= L, for every owned L up to its own
-                const int low = (int)((uint32_t)(k >> 32) & low_mask);
-                int prev = own_lo - 1;
-                if (p > (int)s_bin_start[d]) prev = (int)((uint32_t)(s_keys[p - 1] >> 32) & low_mask);
-                for (int l = max(prev + 1, own_lo); l <= low; l++) seg_start[(d << low_bits) | (uint32_t)l] = (int)dst;
+        for (int i = 0; i < kItems; i++) {
+            const int p = min(i * kSortBlock + tid, in_tile - 1);
+            out_key[i] = s_keys[p];
+            out_value[i] = s_values[p];
+        }
+#pragma unroll
+        for (int i = 0; i < kItems; i++)
+            out_at[i] = s_global[digit_of(out_key[i], shift, mask)] + (uint32_t)(i * kSortBlock + tid);
+#pragma unroll
+        for (int i = 0; i < kItems; i++) {
+            if (i * kSortBlock + tid < in_tile) {
+                keys_out[out_at[i]] = out_key[i];
+                values_out[out_at[i]] = out_value[i];
             }
         }
     }
     if (kTable) {
         if (own_lo <= own_hi) {
+            // the first pair of digit d with a low part >= L, for every owned L up to its own
+            // (a loop of its own: in the one above the LDS reads of all slots are in flight together)
+#pragma unroll 4
+            for (int i = 0; i < kItems; i++) {
+                const int p = i * kSortBlock + tid;
+                if (p >= in_tile) break;
+                const uint32_t field = (uint32_t)(s_keys[p] >> 32);
+                const uint32_t d = (field >> low_bits) & mask;
+                const int low = (int)(field & low_mask);
+                int prev = own_lo - 1;
+                if (p > (int)s_bin_start[d]) prev = (int)((uint32_t)(s_keys[p - 1] >> 32) & low_mask);
+                for (int l = max(prev + 1, own_lo); l <= low; l++)
+                    seg_start[(d << low_bits) | (uint32_t)l] = (int)(s_global[d] + (uint32_t)p);
+            }
             // owned low parts above the last pair of a digit's run: the end of the run
 #pragma unroll
             for (int q = 0; q < kPer; q++) {
