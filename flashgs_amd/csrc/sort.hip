@@ -35,6 +35,7 @@ namespace {
 constexpr int kBins = 256;                      // counters of a counting pass inside a segment (8-bit digits)
 constexpr int kSortBlock = 256;
 constexpr int kSortWaves = kSortBlock / kWave;
+constexpr int kXcds = 8;                        // accelerator dies of the device, workgroup i of a launch runs on die i % 8
 
 // Shape of a partition pass: digits of kBitsT bits, kItemsT pairs per thread.  Up to 65 536 tiles
 // two passes of 8 bits do; above that (an 8K frame has 129 600) digits of 9 bits keep it at two
@@ -305,7 +306,12 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
     const uint32_t mask = (1u << nbits) - 1u;
-    const int tile = blockIdx.x;
+    // Workgroups go round-robin to the 8 XCDs, each with an L2 of its own.  Every XCD takes a
+    // contiguous range of blocks: the runs that neighbouring blocks write for one digit are
+    // neighbours in memory, and the cache line where two of them meet is then completed in one
+    // L2 instead of being written out in parts by two (first pass at 4K: 62 -> 51 us).
+    const int xcd = (int)blockIdx.x % kXcds, per = (int)gridDim.x / kXcds, rest = (int)gridDim.x % kXcds;
+    const int tile = xcd * per + min(xcd, rest) + (int)blockIdx.x / kXcds;
     const int tile_base = tile * kTile;
     const int in_tile = min(kTile, n - tile_base);
 
