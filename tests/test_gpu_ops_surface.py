@@ -36,7 +36,7 @@ def test_rasterizer_forward_matches_oracle(oracle, tile, tmp_path):
     u8, _, _ = oracle.render(c0.width, c0.height, tile[0], tile[1], pre["points_xy"], pre["rgb_depth"],
                              pre["conic_opacity"], vs, rg, bg.numpy(), want_f32=False)
     d = np.abs(img2.astype(np.int16) - u8.astype(np.int16))
-    assert d.max() <= 1 and (d > 0).mean() < 0.01
+    assert d.max() <= 1 and (d > 0).mean() < 0.02
     path = tmp_path / "frame.ppm"
     savePpm(img, str(path))
     data = path.read_bytes()
@@ -148,7 +148,7 @@ def test_render_scene_from_ply_and_cameras_json(oracle, tmp_path, capsys):
         assert data.startswith(head) and len(data) == len(head) + 3 * w * h
         img = np.frombuffer(data[len(head):], np.uint8).reshape(h, w, 3)
         d = np.abs(img.astype(np.int16) - u8.astype(np.int16))
-        assert d.max() <= 1 and (d > 0).mean() < 0.01
+        assert d.max() <= 1 and (d > 0).mean() < 0.02
         assert img.max() > 100          # not an empty frame
 
 
@@ -192,4 +192,4 @@ def test_two_rasterizers_on_two_streams_overlapping(oracle):
     u8, _, _ = oracle.render(c0.width, c0.height, 16, 16, pre["points_xy"], pre["rgb_depth"], pre["conic_opacity"], vs, rg,
                              bg.numpy(), want_f32=False)
     d = np.abs(alone[0].cpu().numpy().astype(np.int16) - u8.astype(np.int16))
-    assert d.max() <= 1 and (d > 0).mean() < 0.01
+    assert d.max() <= 1 and (d > 0).mean() < 0.02

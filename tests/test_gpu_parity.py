@@ -10,6 +10,10 @@ pytestmark = pytest.mark.gpu
 
 IMG_MAX_ABS = 2e-3
 IMG_PSNR_DB = 55.0
+# The colour sums of the blend take weights and colours rounded to f16 (products and sums in fp32):
+# a pixel's colour is within 2^-10 of itself of the oracle's, which moves the few 8-bit values that
+# lie that close to a step of the encode by one.
+IMG_U8_FRACTION = 0.02
 
 
 def _oracle_frame(oracle, sc, cam, capacity, block=(16, 16), bg=(0, 0, 0), sentinel=0.0):
@@ -56,10 +60,13 @@ def _check_frame(oracle, sc, cam, capacity, block=(16, 16), bg=(0, 0, 0)):
     f32 = f32.cpu().numpy()
     err = np.abs(f32 - ref["f32"])
     assert err.max() <= IMG_MAX_ABS, "max abs image error %g" % err.max()
+    # pixel by pixel: the f16 operands of the colour sums cost at most 2^-10 of the colour itself
+    over = err - (2.0 ** -10 * np.abs(ref["f32"]) + 2e-4)
+    assert over.max() <= 0, "a pixel is %g further from the oracle than f16 colour operands explain" % over.max()
     assert gp.psnr(f32, ref["f32"]) > IMG_PSNR_DB
     d8 = np.abs(u8.cpu().numpy().astype(np.int16) - ref["u8"].astype(np.int16))
     assert d8.max() <= 1, "8-bit image differs by more than one step"
-    assert (d8 > 0).mean() < 0.01
+    assert (d8 > 0).mean() < IMG_U8_FRACTION
     return ref
 
 
@@ -467,7 +474,7 @@ def test_blend_long_lists_shared_between_waves(oracle):
                    bg, 0, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
         err = np.abs(out.cpu().numpy() - ref)
-        assert err.max() <= 5e-4, "max abs image error %g" % err.max()
+        assert err.max() <= 1e-3, "max abs image error %g" % err.max()    # 1e-4 (runs) + 2^-10 of a colour
 
 
 def test_ranges_kernel_against_searchsorted():
