@@ -206,6 +206,7 @@ typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 constexpr float kWeightScaleLog2 = 14.0f;
 constexpr float kWeightUnscale = 6.103515625e-05f;          // 2^-14
+constexpr float kColourMax = 65504.0f;                      // largest f16: a colour beyond it is drawn as this
 
 // A read that stays where it is written: the compiler neither sinks it to its first use nor drops
 // it when the value turns out unused (volatile on the vector type keeps it one wide LDS read).
@@ -372,7 +373,8 @@ __device__ __forceinline__ bool walk_list(
             const float e = stage_g ? ey + (float)(kGy / 2) : ex + (float)(kFx / 2);
             const float curv = unused ? 0.0f : (stage_g ? nco.z : nco.x);
             const float lin = unused ? 0.0f : nco.y * (stage_g ? ex : ey);
-            const float con = stage_g ? 0.0f : (unused ? -1.0e30f : (nco.w + kWeightScaleLog2) - (nco.y * ex) * ey);
+            // (log2 of the opacity is held below 2 so that no scaled weight leaves f16's range)
+            const float con = stage_g ? 0.0f : (unused ? -1.0e30f : ((nco.w > 1.99f ? 1.99f : nco.w) + kWeightScaleLog2) - (nco.y * ex) * ey);
             const float c0 = con + e * (curv * e + lin);
             const float c1 = -(2.0f * curv * e + lin);
 #pragma unroll
@@ -386,9 +388,12 @@ __device__ __forceinline__ bool walk_list(
             if (stage_g) {
                 stage_group[stage_slot & 3] = unused ? 0.0f : nco.y;
                 _Float16* const colour = reinterpret_cast<_Float16*>(stage_group + 4) + (stage_slot & 3);
-                colour[0] = (_Float16)nrgb.x;
-                colour[4] = (_Float16)nrgb.y;
-                colour[8] = (_Float16)nrgb.z;
+                auto in_range = [](float c) {           // NaN stays NaN
+                    return c > kColourMax ? kColourMax : (c < -kColourMax ? -kColourMax : c);
+                };
+                colour[0] = (_Float16)in_range(nrgb.x);
+                colour[4] = (_Float16)in_range(nrgb.y);
+                colour[8] = (_Float16)in_range(nrgb.z);
                 colour[12] = (_Float16)0.0f;
             }
         }
