@@ -109,6 +109,9 @@ size_t fgs_get_sort_buffer_size(int num_rendered);
  * csrc/cuda_rasterizer/render.cu:549-608): zero `ranges`, find each tile's [start,end) in the
  * sorted keys, blend front to back and write out_color u8[H,W,3].  `ranges` int32[tiles,2] is
  * scratch that holds the tile ranges afterwards.  bg_color is a host array of 3 floats.
+ * Exponent, alpha and transmittance are fp32; the colour sums take the weights alpha*T and the
+ * colours rounded to f16 (products and sums in fp32), so a pixel's colour is within 2^-10 of
+ * itself of the all-fp32 sum; colours beyond +-65504 are drawn as +-65504.
  * A frame of at most 8192 16x16 tiles first ranks its tiles by list length into a table the
  * library keeps per (device, stream) (32 KB, allocated on the first such call on that stream),
  * and the rest of a list of more than 768 entries is blended in four runs that each stop on
