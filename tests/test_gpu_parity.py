@@ -477,6 +477,68 @@ def test_blend_long_lists_shared_between_waves(oracle):
         assert err.max() <= 1e-3, "max abs image error %g" % err.max()    # 1e-4 (runs) + 2^-10 of a colour
 
 
+def _blend_lists(oracle, lists, W, H, bg, seed, colour_hi=1.5):
+    """Builds the attribute tensors and ranges for hand-made per-tile lists (tile, length, opacity),
+    blends them with fgs_blend and with the oracle; returns (GPU float image, oracle float image)."""
+    import gpu_pipeline as gp
+    from flashgs_amd import cabi
+    import torch
+    gx, gy = (W + 15) // 16, (H + 15) // 16
+    rng = np.random.default_rng(seed)
+    xy, co, rgbd, ranges = [], [], [], np.zeros((gx * gy, 2), np.int32)
+    at = 0
+    for t, n, op in sorted(lists):
+        tx, ty = t % gx, t // gx
+        c = np.stack([tx * 16 + rng.uniform(-4, 20, n), ty * 16 + rng.uniform(-4, 20, n)], 1)
+        sig = rng.uniform(3.0, 12.0, (n, 2))
+        rho = rng.uniform(-0.6, 0.6, n)
+        det = (sig[:, 0] * sig[:, 1]) ** 2 * (1 - rho ** 2)
+        cx, cz = sig[:, 1] ** 2 / det, sig[:, 0] ** 2 / det
+        cy = -rho * sig[:, 0] * sig[:, 1] / det
+        log2e = 1.4426950408889634
+        xy.append(c)
+        co.append(np.stack([-0.5 * log2e * cx, -log2e * cy, -0.5 * log2e * cz, np.log2(np.full(n, op))], 1))
+        rgbd.append(np.concatenate([rng.uniform(0, colour_hi, (n, 3)), rng.uniform(1, 50, (n, 1))], 1))
+        ranges[t] = (at, at + n)
+        at += n
+    xy = np.concatenate(xy).astype(np.float32)
+    co = np.concatenate(co).astype(np.float32)
+    rgbd = np.concatenate(rgbd).astype(np.float32)
+    vals = np.arange(at, dtype=np.uint32)
+    bg = np.asarray(bg, np.float32)
+    _, ref, _ = oracle.render(W, H, 16, 16, xy, rgbd, co, vals, ranges, bg, want_u8=False)
+    out = torch.full((H, W, 3), -1.0, device=gp.DEV, dtype=torch.float32)
+    d = [gp.dev(a) for a in (xy, rgbd, co)]
+    dv, dr = gp.dev(vals.view(np.int32)), gp.dev(ranges)
+    cabi.blend(16, 16, W, H, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), dv.data_ptr(), dr.data_ptr(),
+               bg, 0, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return out.cpu().numpy(), ref
+
+
+@pytest.mark.parametrize("W,H", [(320, 240), (3840, 400)])       # the kernel of small frames and the one of large frames
+def test_blend_faint_weights_keep_their_relative_accuracy(oracle, W, H):
+    """The colour sums take their weights as f16.  Lists of thousands of Gaussians whose weights
+    alpha*T lie between 1e-8 and 1e-5, far below f16's smallest normal number 6e-5, still add up to
+    colours that are right to 2^-10 of themselves: the weights are scaled before the conversion."""
+    gx = (W + 15) // 16
+    lists = [(t, 1500 + 37 * (t % 5), op) for t, op in zip(range(0, 12 * gx, gx + 3), [1e-5, 3e-6, 1e-6, 3e-7, 1e-7, 1e-8] * 2)]
+    got, ref = _blend_lists(oracle, lists, W, H, (0.0, 0.0, 0.0), seed=5)
+    lit = ref > 0
+    assert lit.any() and ref[lit].max() < 0.05                      # faint sums, nothing near 1
+    assert np.all(np.abs(got - ref)[lit] <= 2.0 ** -10 * ref[lit] + 1e-9)
+    assert np.all(got[~lit] == 0)
+
+
+def test_blend_colours_up_to_the_f16_range(oracle):
+    """Colours far above 1 (up to 6e4, just inside f16) blend like any other: within 2^-10 of the
+    pixel's own colour."""
+    lists = [(t, 40 + t, 0.3) for t in range(0, 300, 7)]
+    got, ref = _blend_lists(oracle, lists, 320, 240, (0.1, 0.2, 0.3), seed=9, colour_hi=6.0e4)
+    assert ref.max() > 1.0e4
+    assert np.all(np.abs(got - ref) <= 2.0 ** -10 * np.abs(ref) + 1e-4)
+
+
 def test_ranges_kernel_against_searchsorted():
     import gpu_pipeline as gp
     import torch
