@@ -388,8 +388,8 @@ __device__ __forceinline__ bool walk_list(
             if (stage_g) {
                 stage_group[stage_slot & 3] = unused ? 0.0f : nco.y;
                 _Float16* const colour = reinterpret_cast<_Float16*>(stage_group + 4) + (stage_slot & 3);
-                auto in_range = [](float c) {           // NaN stays NaN
-                    return c > kColourMax ? kColourMax : (c < -kColourMax ? -kColourMax : c);
+                auto in_range = [&](float c) {          // NaN stays NaN; a slot past the end of the list holds no colour
+                    return unused ? 0.0f : (c > kColourMax ? kColourMax : (c < -kColourMax ? -kColourMax : c));
                 };
                 colour[0] = (_Float16)in_range(nrgb.x);
                 colour[4] = (_Float16)in_range(nrgb.y);
