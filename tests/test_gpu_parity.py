@@ -118,6 +118,51 @@ def test_wide_tiles_on_a_frame_with_many_tiles(oracle, block):
     _check_frame(oracle, sc, cam, 1 << 22, block=block, bg=(0.1, 0.2, 0.3))
 
 
+def test_random_frames_with_odd_sizes_and_cameras(oracle):
+    """Twenty random frames: 1 to 150 000 Gaussians, images from 1x1 to 4000x1080 including sizes
+    one below and one above a tile, fields of view from 10 to 120 degrees, cameras inside and
+    outside the cloud, all three tile shapes.  Keys, values, their order, the attribute records,
+    the sorted lists and the ranges are compared bit for bit, the image within the tolerance."""
+    import gpu_pipeline as gp
+    for seed in range(20):
+        rng = np.random.default_rng(1000 + seed)
+        n = int(rng.choice([1, 7, 63, 257, 5000, 40000, 150000]))
+        sc = scenes.config0(n=n)
+        sc.position = (sc.position * rng.uniform(0.2, 3.0)).astype(np.float32)
+        ls = rng.normal(rng.uniform(-5, -1.0), rng.uniform(0.3, 1.5), (n, 3))
+        sc.cov3d = scenes.cov3d_from_scale_rotation(np.exp(ls).astype(np.float32), scenes._unit_quats(rng, n))
+        W = int(rng.choice([1, 15, 16, 17, 100, 333, 640, 1280, 1921, 4000]))
+        H = int(rng.choice([1, 16, 31, 200, 360, 721, 1080]))
+        cam = scenes.look_at(rng.uniform(-6, 6, 3), rng.uniform(-2, 2, 3), W, H, rng.uniform(10, 120))
+        block = [(16, 16), (32, 16), (32, 32)][seed % 3]
+        bg = rng.uniform(0, 1, 3).astype(np.float32)
+        cap = 1 << 24
+        r = oracle.preprocess(sc.position, sc.shs, sc.opacity, sc.cov3d, W, H, block[0], block[1], cam.position, cam.rotation,
+                              cam.focal_x, cam.focal_y, cam.zFar, cam.zNear, cap)
+        K = r["num_rendered"]
+        assert r["rc"] == 0 and K <= cap
+        where = "seed %d: %d Gaussians, %dx%d, tile %s, %d pairs" % (seed, n, W, H, block, K)
+        got = gp.preprocess(gp.SceneOnDevice(sc), cam, cap, block=block)
+        assert got["num_rendered"] == K, where
+        assert np.array_equal(gp.u64(got["keys"])[:K], r["keys"][:K]), where
+        assert np.array_equal(gp.u32(got["values"])[:K], r["values"][:K]), where
+        vis = np.zeros(n, bool)
+        vis[r["values"][:K]] = True
+        for name in ("points_xy", "conic_opacity", "rgb_depth"):
+            assert np.array_equal(gp.bits(got[name].cpu().numpy()[vis]), gp.bits(r[name][vis])), where + ", " + name
+        ks, vs = oracle.sort(K, W, H, block[0], block[1], r["keys"][:K], r["values"][:K])
+        gks, gvs = gp.sort(K, W, H, got["keys"], got["values"], block)
+        assert np.array_equal(gp.u64(gks)[:K], ks) and np.array_equal(gp.u32(gvs)[:K], vs), where
+        gx, gy = (W + block[0] - 1) // block[0], (H + block[1] - 1) // block[1]
+        rg = oracle.ranges(K, ks, gx * gy)
+        _, ref, _ = oracle.render(W, H, block[0], block[1], r["points_xy"], r["rgb_depth"], r["conic_opacity"], vs, rg, bg,
+                                  want_u8=False)
+        grg, _, f32 = gp.render(K, W, H, got["points_xy"], got["rgb_depth"], got["conic_opacity"], gks, gvs, bg, block)
+        assert np.array_equal(grg.cpu().numpy(), rg), where
+        err = np.abs(f32.cpu().numpy() - ref).max()
+        assert err <= IMG_MAX_ABS, where + ": max abs image error %g" % err
+
+
 def test_degenerate_inputs_match_the_oracle(oracle):
     """NaN / infinite / zero / enormous entries in every input tensor: the kernels must neither fault
     nor disagree with the oracle about which keys such Gaussians emit (the float->int conversions
