@@ -496,6 +496,9 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
         return;
     }
     const int ticket = (int)blockIdx.x - 1;
+    // Every later workgroup's offset waits for this one's count: until the count is published the
+    // waves ask for a higher issue priority than the waves that are past that point.
+    __builtin_amdgcn_s_setprio(2);
     const int idx = ticket * kBlock + tid;
     // tile coordinates travel in 12 bits each and tile indices in 26 when candidates are laid flat
     const bool pack_ok = cam.gx <= 4096 && cam.gy <= 4096 && (long long)cam.gx * cam.gy <= (1 << 26);
@@ -829,6 +832,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     // The workgroup's count is published right away; its offset is picked up after the colour
     // work below, when the scanner has long written it.
     if (tid == 0) publish(counts + ticket, pack_status(kStateCount, block_total));
+    __builtin_amdgcn_s_setprio(0);
 
     // ---- attributes of Gaussians that emit a key, and of every Gaussian whose rectangle is a
     // single tile, hit or not (preprocess.cu:317, 411-417: vertex_valid starts as single_tile) ----
