@@ -352,7 +352,7 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
         for (int q = 0; q < kPer; q++) {
             const int d = q * kSortBlock + tid;
             total[q] = 0; before[q] = 0;
-#pragma unroll 8
+#pragma unroll 16
             for (int b = 0; b < raw_rows; b++) {
                 const uint32_t c = start[(size_t)b * kB + d];
                 total[q] += c;
