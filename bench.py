@@ -355,7 +355,10 @@ def main():
         "value": head["fps"], "unit": "frames/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms_per_frame"], "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f32",
+        "dtype_note": "fp32 throughout (ndc2Pix fp64 as the reference); the blend's colour sums take f16 operands "
+                      "(weights alpha*T, colours) with fp32 products and accumulation, within 2^-10 of a pixel's colour",
+        "data": "synthetic",
         "config": {"workload": head["workload"], "gaussians": head["gaussians"], "width": head["width"], "height": head["height"],
                    "tile": "16x16", "sh_degree": 3, "pairs": head["pairs"], "poses": head["poses"]},
         "target_fps": 400 if args.config == 2 else None,
