@@ -314,6 +314,13 @@ def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops):
                                  stages_ms_mean={k: round(v, 4) for k, v in traj_stage.items()})
     if with_ops:
         rep["ops_surface_ms_per_frame"], rep["ops_surface_image_identical"] = ops_surface_ms(torch, np, fr, steps)
+        # the same frame with the colour sums by fp32 multiply-add instead of the matrix unit (fgs_set_colour_sums)
+        prev = cabi.set_colour_sums(cabi.COLOUR_SUMS_FP32)
+        try:
+            ms32, stage32, _, _ = fr.timed(fr.cams[:1], max(5, steps // 2), 2, False)
+        finally:
+            cabi.set_colour_sums(prev)
+        rep["fp32_colour_sums"] = dict(ms_per_frame=round(ms32, 4), blend_ms=round(stage32["blend"], 4))
     return rep, fr
 
 
@@ -362,6 +369,7 @@ def main():
         "config": {"workload": head["workload"], "gaussians": head["gaussians"], "width": head["width"], "height": head["height"],
                    "tile": "16x16", "sh_degree": 3, "pairs": head["pairs"], "poses": head["poses"]},
         "target_fps": 400 if args.config == 2 else None,
+        "fp32_colour_sums": head.get("fp32_colour_sums"),
         "stages": head["stages"],
         "roofline": head["roofline"],
         "cpu_baseline": head["cpu_baseline"],

@@ -33,6 +33,7 @@ SIGNATURES = {
     "fgs_blend_kernel_name": (C.c_char_p, [C.c_int] * 4),
     "fgs_camera_matrices": (None, [C.c_void_p] * 2 + [C.c_int] * 2 + [C.c_float] * 4 + [C.c_void_p] * 2),
     "fgs_set_scan_spin_limit": (C.c_uint, [C.c_uint]),
+    "fgs_set_colour_sums": (C.c_int, [C.c_int]),
     "fgs_last_error": (C.c_char_p, []),
     "fgs_abi_version": (C.c_int, []),
 }
@@ -91,6 +92,18 @@ def preprocess(P, positions, shs, opacities, cov3ds, width, height, block_x, blo
                                points_xy, rgb_depth, conic_opacity, keys, values, curr_offset,
             key_capacity, stream)
     _check(rc, "fgs_preprocess_static" if static else "fgs_preprocess")
+
+
+COLOUR_SUMS_MATRIX_F16, COLOUR_SUMS_FP32 = 0, 1
+
+
+def set_colour_sums(mode):
+    """How later blends form their colour sums (matrix unit with f16 operands, or fp32 multiply-add);
+    returns the previous mode."""
+    prev = int(load().fgs_set_colour_sums(int(mode)))
+    if prev < 0:
+        raise RuntimeError("fgs_set_colour_sums failed: %s" % last_error())
+    return prev
 
 
 def set_scan_spin_limit(polls):

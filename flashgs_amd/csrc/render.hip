@@ -13,6 +13,7 @@
 // workgroup is a single wave, so no workgroup barrier is needed anywhere.
 #include "fgs_internal.h"
 
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -252,6 +253,24 @@ __device__ __forceinline__ void shade_quad(Quad& q, const float xy[2][2], const 
         }
 }
 
+// The all-fp32 form (render.cu:40-52 operation for operation): colour sums by multiply-add.
+__device__ __forceinline__ void shade_quad_fp32(Quad& q, const float xy[2][2], const float2 f, const float2 g, const float cy,
+                                                const float4 rgb)
+{
+    const float fx[2] = {f.x, f.y}, gy[2] = {g.x, g.y};
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const float alpha = __builtin_amdgcn_exp2f(__builtin_fmaf(cy, xy[j][i], fx[i] + gy[j]));
+            const float at = alpha * q.T[j][i];
+            q.r[j][i] += rgb.x * at;
+            q.g[j][i] += rgb.y * at;
+            q.b[j][i] += rgb.z * at;
+            q.T[j][i] -= at;
+        }
+}
+
 __device__ __forceinline__ uint32_t pack_f16(float a, float b)
 {
     const float2_t v = {a, b};
@@ -265,9 +284,9 @@ struct LaneRole {
     static constexpr int kFx = 16 * SX, kGy = 16 * SY;
     static constexpr int kRec = kFx + kGy + 4;  // floats per staged Gaussian: F table, G table; padded so that the
                                                 // staging lanes, one record apart, write to different LDS banks
-    static constexpr int kGroupRec = 12;        // floats per group of four: cy x 4, then 4 channels x 4 f16
+    static constexpr int kGroupRec = 28;        // floats per group of four: cy x 4, 4 channels x 4 f16, (r, g, b, -) x 4 as fp32
     static constexpr int kStage = kBatch * kRec + kGroups * kGroupRec;      // floats of a wave's staging area
-    uint32_t off_f, off_g, off_cy, off_colour;  // byte offsets into the staging area
+    uint32_t off_f, off_g, off_cy, off_colour;  // byte offsets into the staging area (fp32 colours: off_cy + 48)
     int stage_slot;                             // Gaussian lane%32 of the batch
     bool stage_g;                               // lanes 0-31 tabulate F, 32-63 G
     float xy[SX * SY][2][2];                    // X*Y of the quad's pixels, offsets from the tile centre
@@ -311,7 +330,7 @@ __device__ __forceinline__ void clear_quad(Quad& q)
 // distance from the start of the tile's list, so that the pairs are the reference's pairs.
 // Returns true when the walk ended at the tile-wide stop.  s_rec is this wave's staging area of
 // LaneRole::kStage floats.
-template <int SX, int SY>
+template <int SX, int SY, bool kFp32>
 __device__ __forceinline__ bool walk_list(
     const LaneRole<SX, SY>& role, float* s_rec,
     const uint32_t* __restrict__ point_list, int begin, int n,
@@ -374,7 +393,8 @@ __device__ __forceinline__ bool walk_list(
             const float curv = unused ? 0.0f : (stage_g ? nco.z : nco.x);
             const float lin = unused ? 0.0f : nco.y * (stage_g ? ex : ey);
             // (log2 of the opacity is held below 2 so that no scaled weight leaves f16's range)
-            const float con = stage_g ? 0.0f : (unused ? -1.0e30f : ((nco.w > 1.99f ? 1.99f : nco.w) + kWeightScaleLog2) - (nco.y * ex) * ey);
+            const float w_log2 = kFp32 ? nco.w : (nco.w > 1.99f ? 1.99f : nco.w) + kWeightScaleLog2;
+            const float con = stage_g ? 0.0f : (unused ? -1.0e30f : w_log2 - (nco.y * ex) * ey);
             const float c0 = con + e * (curv * e + lin);
             const float c1 = -(2.0f * curv * e + lin);
 #pragma unroll
@@ -391,10 +411,15 @@ __device__ __forceinline__ bool walk_list(
                 auto in_range = [&](float c) {          // NaN stays NaN; a slot past the end of the list holds no colour
                     return unused ? 0.0f : (c > kColourMax ? kColourMax : (c < -kColourMax ? -kColourMax : c));
                 };
-                colour[0] = (_Float16)in_range(nrgb.x);
-                colour[4] = (_Float16)in_range(nrgb.y);
-                colour[8] = (_Float16)in_range(nrgb.z);
-                colour[12] = (_Float16)0.0f;
+                if (!kFp32) {
+                    colour[0] = (_Float16)in_range(nrgb.x);
+                    colour[4] = (_Float16)in_range(nrgb.y);
+                    colour[8] = (_Float16)in_range(nrgb.z);
+                    colour[12] = (_Float16)0.0f;
+                }
+                if (kFp32)
+                    *reinterpret_cast<float4*>(stage_group + 12 + 4 * (stage_slot & 3)) =
+                        unused ? make_float4(0.f, 0.f, 0.f, 0.f) : make_float4(nrgb.x, nrgb.y, nrgb.z, 0.f);
             }
         }
         __builtin_amdgcn_wave_barrier();
@@ -415,22 +440,31 @@ __device__ __forceinline__ bool walk_list(
         auto fetch_group = [&](int g) {
             StagedGroup r;
             r.cy = lds_read<float4>(rec_bytes + off_cy + g * kGroupRec * 4);
-            r.colour = lds_read<float2>(rec_bytes + off_colour + g * kGroupRec * 4);
+            r.colour = kFp32 ? make_float2(0.f, 0.f) : lds_read<float2>(rec_bytes + off_colour + g * kGroupRec * 4);
             return r;
         };
         uint32_t packed[kSub][4][2];        // f16 weights of the group's Gaussians 0-1 and 2-3, per pixel
         float w0[kSub][4], w1[kSub][4];
-        auto shade = [&](const Staged& r, float cy, float (&w)[kSub][4]) {
+        auto shade = [&](const Staged& r, float cy, float (&w)[kSub][4], const float4& rgb) {
 #pragma unroll
-            for (int s = 0; s < kSub; s++) shade_quad(quad[s], role.xy[s], r.f[s % SX], r.g[s / SX], cy, w[s]);
+            for (int s = 0; s < kSub; s++) {
+                if (kFp32) shade_quad_fp32(quad[s], role.xy[s], r.f[s % SX], r.g[s / SX], cy, rgb);
+                else shade_quad(quad[s], role.xy[s], r.f[s % SX], r.g[s / SX], cy, w[s]);
+            }
+        };
+        // fp32 colours of Gaussian k of group g (the same address in every lane)
+        auto fetch_rgb = [&](int g, int k) {
+            return kFp32 ? lds_read<float4>(rec_bytes + off_cy + g * kGroupRec * 4 + 48 + 16 * k) : make_float4(0.f, 0.f, 0.f, 0.f);
         };
         auto pack = [&](int half) {
+            if (kFp32) return;
 #pragma unroll
             for (int s = 0; s < kSub; s++)
 #pragma unroll
                 for (int p = 0; p < 4; p++) packed[s][p][half] = pack_f16(w0[s][p], w1[s][p]);
         };
         auto accumulate = [&](const StagedGroup& grp) {
+            if (kFp32) return;
             const half4_t colour = __builtin_bit_cast(half4_t, grp.colour);
 #pragma unroll
             for (int s = 0; s < kSub; s++)
@@ -454,17 +488,19 @@ __device__ __forceinline__ bool walk_list(
         if (4 * (G) >= cnt) break;                                                           \
         grp = next_grp;                                                                      \
         next_grp = fetch_group(((G) + 1) % kGroups);    /* past the batch: read and dropped */\
+        rgb0 = fetch_rgb(G, 0); rgb1 = fetch_rgb(G, 1);                                      \
         second = fetch(4 * (G) + 1);                                                         \
-        shade(first, grp.cy.x, w0);                                                          \
+        shade(first, grp.cy.x, w0, rgb0);                                                    \
         first = fetch(4 * (G) + 2);                                                          \
-        shade(second, grp.cy.y, w1);                                                         \
+        shade(second, grp.cy.y, w1, rgb1);                                                   \
         pack(0);                                                                             \
-        stop_mid = all_stopped();                                                             \
+        stop_mid = all_stopped();                                                            \
         if (!stop_mid) {                                                                     \
+            rgb0 = fetch_rgb(G, 2); rgb1 = fetch_rgb(G, 3);                                  \
             second = fetch(4 * (G) + 3);                                                     \
-            shade(first, grp.cy.z, w0);                                                      \
+            shade(first, grp.cy.z, w0, rgb0);                                                \
             first = fetch((4 * (G) + 4) % kBatch);                                           \
-            shade(second, grp.cy.w, w1);                                                     \
+            shade(second, grp.cy.w, w1, rgb1);                                               \
             pack(1);                                                                         \
         } else {                                                                             \
             _Pragma("unroll") for (int s = 0; s < kSub; s++)                                 \
@@ -472,9 +508,10 @@ __device__ __forceinline__ bool walk_list(
         }                                                                                    \
         accumulate(grp);                                                                     \
         if (stop_mid || all_stopped()) { done = true; break; }
+        static_assert(kBatch == 32, "the groups below cover a batch of 32");
         Staged first = fetch(0), second;
         StagedGroup grp, next_grp = fetch_group(0);
-        static_assert(kBatch == 32, "the groups below cover a batch of 32");
+        float4 rgb0, rgb1;
         bool stop_mid = false;
         do {
             FGS_GROUP(0) FGS_GROUP(1) FGS_GROUP(2) FGS_GROUP(3) FGS_GROUP(4) FGS_GROUP(5) FGS_GROUP(6) FGS_GROUP(7)
@@ -488,7 +525,7 @@ __device__ __forceinline__ bool walk_list(
     static_assert(Role::kStage >= 16 * 68, "the staging area holds the 64 x 16 colour sums of a sub-tile");
     const int lane = lane_id();
 #pragma unroll
-    for (int s = 0; s < kSub; s++) {
+    for (int s = 0; s < (kFp32 ? 0 : kSub); s++) {
         __builtin_amdgcn_wave_barrier();
         char* const out = reinterpret_cast<char*>(s_rec) + 4 * ((lane >> 2) * 68 + (lane & 3));
 #pragma unroll
@@ -557,7 +594,7 @@ __device__ __forceinline__ bool tile_of_position(int group, int tiles_x, int til
     return *tile_x < tiles_x && *tile_y < tiles_y;
 }
 
-template <int SX, int SY>
+template <int SX, int SY, bool kFp32>
 __device__ __forceinline__ void blend_tile(
     const int2* __restrict__ ranges,
     const uint32_t* __restrict__ point_list,
@@ -591,7 +628,7 @@ __device__ __forceinline__ void blend_tile(
 #pragma unroll
     for (int s = 0; s < kSub; s++) clear_quad(quad[s]);
     const float centre_x = (float)(tile_x * kFx + kFx / 2), centre_y = (float)(tile_y * kGy + kGy / 2);
-    walk_list<SX, SY>(role, s_rec, point_list, range.x, n, centre_x, centre_y, points_xy, rgb_depth, conic_opacity, quad);
+    walk_list<SX, SY, kFp32>(role, s_rec, point_list, range.x, n, centre_x, centre_y, points_xy, rgb_depth, conic_opacity, quad);
     write_tile<SX, SY>(lane, tile_x, tile_y, width, height, quad, bg_r, bg_g, bg_b, out_u8, out_f32);
 }
 
@@ -612,10 +649,10 @@ constexpr int kFewWaves = SX * SY == 1 ? 4 : SX * SY == 2 ? 3 : 2;
 template <int SX, int SY>
 constexpr int kPlainWaves = SX * SY == 1 ? 6 : kFewWaves<SX, SY>;
 
-template <int SX, int SY>
+template <int SX, int SY, bool kFp32>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(kPlainWaves<SX, SY>))) void blend_kernel(FGS_BLEND_PARAMS)
 {
-    blend_tile<SX, SY>(FGS_BLEND_ARGS);
+    blend_tile<SX, SY, kFp32>(FGS_BLEND_ARGS);
 }
 
 // The same kernel held to 4 resident waves per SIMD (16 per CU; 3 and 2 for the wider tiles,
@@ -623,10 +660,10 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(kPlainWav
 // lists of the tiles in flight compete for the 4 MB L2 of their XCD: when there are more tiles
 // than the chip holds at once, fewer resident waves mean fewer misses (a 4K frame takes the same
 // time at 4, 5 and 6 waves per SIMD and half as long again at 8).
-template <int SX, int SY>
+template <int SX, int SY, bool kFp32>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(kFewWaves<SX, SY>, kFewWaves<SX, SY>))) void blend_kernel_few_waves(FGS_BLEND_PARAMS)
 {
-    blend_tile<SX, SY>(FGS_BLEND_ARGS);
+    blend_tile<SX, SY, kFp32>(FGS_BLEND_ARGS);
 }
 
 // A frame of few tiles is placed on the chip almost at once, one wave per tile: the launch then
@@ -644,6 +681,7 @@ constexpr int kOwnShare = 256;
 constexpr int kMinRest = 512;               // a shorter rest is not worth two barriers: the owner walks it
 constexpr int kSharedWaves = 4;
 
+template <bool kFp32>
 __global__ __launch_bounds__(kSharedWaves * kWave) __attribute__((amdgpu_waves_per_eu(6, 6))) void blend_kernel_shared(FGS_BLEND_PARAMS, const uint32_t* __restrict__ tile_order)
 {
     using Role = LaneRole<1, 1>;
@@ -692,7 +730,7 @@ __global__ __launch_bounds__(kSharedWaves * kWave) __attribute__((amdgpu_waves_p
             count = min(run, rest - skip);
         }
         clear_quad(part[0]);
-        const bool stopped = walk_list<1, 1>(role, s_rec[wave], point_list, __builtin_amdgcn_readfirstlane(s_from[v]) + skip, count,
+        const bool stopped = walk_list<1, 1, kFp32>(role, s_rec[wave], point_list, __builtin_amdgcn_readfirstlane(s_from[v]) + skip, count,
                                              (float)(__builtin_amdgcn_readfirstlane(s_tile_x[v]) * 16 + 8),
                                              (float)(__builtin_amdgcn_readfirstlane(s_tile_y[v]) * 16 + 8),
                                              points_xy, rgb_depth, conic_opacity, part);
@@ -744,6 +782,9 @@ __global__ __launch_bounds__(kSharedWaves * kWave) __attribute__((amdgpu_waves_p
 }
 #undef FGS_BLEND_PARAMS
 #undef FGS_BLEND_ARGS
+
+// How the colour sums are formed, for every blend launched after the setting (see fgs_set_colour_sums).
+std::atomic<int> g_colour_sums{FGS_COLOUR_SUMS_MATRIX_F16};
 
 int check_tile(int block_x, int block_y, int* sx, int* sy, const char* who)
 {
@@ -826,9 +867,11 @@ int blend_impl(int block_x, int block_y, int width, int height,
     rc = blend_shape(block_x, block_y, tiles_x, tiles_y, &shape);
     if (rc != FGS_OK) return rc;
     const bool few_waves = shape.few_waves;
+    const bool fp32 = g_colour_sums.load() == FGS_COLOUR_SUMS_FP32;
 #define FGS_LAUNCH_BLEND(SX, SY)                                                                        \
     do {                                                                                                \
-        auto kernel = few_waves ? blend_kernel_few_waves<SX, SY> : blend_kernel<SX, SY>;                \
+        auto kernel = fp32 ? (few_waves ? blend_kernel_few_waves<SX, SY, true> : blend_kernel<SX, SY, true>) \
+                           : (few_waves ? blend_kernel_few_waves<SX, SY, false> : blend_kernel<SX, SY, false>); \
         hipLaunchKernelGGL(kernel, grid, dim3(kWave), 0, st,                                            \
                            (const int2*)ranges, values_sorted, width, height, tiles_x, tiles_y,         \
                            (const float2*)points_xy, (const float4*)rgb_depth, (const float4*)conic_opacity, \
@@ -840,7 +883,7 @@ int blend_impl(int block_x, int block_y, int width, int height,
         rc = tile_order_table(st, &tile_order);
         if (rc != FGS_OK) return rc;
         hipLaunchKernelGGL(tile_order_kernel, dim3(1), dim3(1024), 0, st, (const int2*)ranges, num_tiles, tile_order);
-        hipLaunchKernelGGL(blend_kernel_shared, dim3((unsigned)((num_tiles + kSharedWaves - 1) / kSharedWaves)), dim3(kSharedWaves * kWave), 0, st,
+        hipLaunchKernelGGL(fp32 ? blend_kernel_shared<true> : blend_kernel_shared<false>, dim3((unsigned)((num_tiles + kSharedWaves - 1) / kSharedWaves)), dim3(kSharedWaves * kWave), 0, st,
                            (const int2*)ranges, values_sorted, width, height, tiles_x, tiles_y,
                            (const float2*)points_xy, (const float4*)rgb_depth, (const float4*)conic_opacity,
                            bg[0], bg[1], bg[2], out_u8, out_f32, (const uint32_t*)tile_order);
@@ -897,6 +940,15 @@ extern "C" int fgs_render_f32(int block_x, int block_y, int num_rendered, int wi
                             out_color_u8, out_color_f32, stream, "fgs_render_f32");
 }
 
+extern "C" int fgs_set_colour_sums(int mode)
+{
+    if (mode != FGS_COLOUR_SUMS_MATRIX_F16 && mode != FGS_COLOUR_SUMS_FP32) {
+        fgs::fail(FGS_E_INVALID, "fgs_set_colour_sums: mode %d unknown", mode);
+        return -1;
+    }
+    return fgs::g_colour_sums.exchange(mode);
+}
+
 extern "C" const char* fgs_blend_kernel_name(int block_x, int block_y, int width, int height)
 {
     using namespace fgs;
@@ -904,10 +956,13 @@ extern "C" const char* fgs_blend_kernel_name(int block_x, int block_y, int width
     if (check_tile(block_x, block_y, &sx, &sy, "fgs_blend_kernel_name") != FGS_OK || width <= 0 || height <= 0) return "";
     BlendShape shape;
     if (blend_shape(block_x, block_y, (width + block_x - 1) / block_x, (height + block_y - 1) / block_y, &shape) != FGS_OK) return "";
-    if (shape.shared) return "tile_order_kernel + blend_kernel_shared";
-    if (sx == 1 && sy == 1) return shape.few_waves ? "blend_kernel_few_waves<1, 1>" : "blend_kernel<1, 1>";
-    if (sx == 2 && sy == 1) return shape.few_waves ? "blend_kernel_few_waves<2, 1>" : "blend_kernel<2, 1>";
-    return shape.few_waves ? "blend_kernel_few_waves<2, 2>" : "blend_kernel<2, 2>";
+    const bool fp32 = g_colour_sums.load() == FGS_COLOUR_SUMS_FP32;
+#define FGS_NAME(few, plain) (shape.few_waves ? (fp32 ? few ", true>" : few ", false>") : (fp32 ? plain ", true>" : plain ", false>"))
+    if (shape.shared) return fp32 ? "tile_order_kernel + blend_kernel_shared<true>" : "tile_order_kernel + blend_kernel_shared<false>";
+    if (sx == 1 && sy == 1) return FGS_NAME("blend_kernel_few_waves<1, 1", "blend_kernel<1, 1");
+    if (sx == 2 && sy == 1) return FGS_NAME("blend_kernel_few_waves<2, 1", "blend_kernel<2, 1");
+    return FGS_NAME("blend_kernel_few_waves<2, 2", "blend_kernel<2, 2");
+#undef FGS_NAME
 }
 
 extern "C" int fgs_tile_ranges(int block_x, int block_y, int num_rendered, int width, int height,

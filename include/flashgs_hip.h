@@ -167,6 +167,21 @@ int fgs_blend(int block_x, int block_y, int width, int height,
 const char* fgs_blend_kernel_name(int block_x, int block_y, int width, int height);
 
 /*
+ * No counterpart in the reference.  How the blend forms its colour sums C += (alpha T) c, for
+ * every blend launched after the call (process-wide); returns the previous mode, -1 for an
+ * unknown one.
+ *   FGS_COLOUR_SUMS_MATRIX_F16 (default): on the matrix unit; the weights alpha T and the colours
+ *     are rounded to f16, products and sums are fp32: a pixel's colour is within 2^-10 of itself
+ *     of the all-fp32 sum, colours beyond +-65504 are drawn as +-65504.
+ *   FGS_COLOUR_SUMS_FP32: by fp32 multiply-add, operation for operation what render.cu:40-52
+ *     does; about a tenth slower on a 4K frame.
+ * Exponent, alpha and transmittance are fp32 in both.
+ */
+#define FGS_COLOUR_SUMS_MATRIX_F16 0
+#define FGS_COLOUR_SUMS_FP32       1
+int fgs_set_colour_sums(int mode);
+
+/*
  * Host-side camera set-up used by fgs_preprocess (preprocess.cu:420-448,461-466), exposed so
  * callers and tests can inspect it: column-major 4x4 view and projection matrices.
  */

@@ -76,3 +76,15 @@ def test_bad_arguments_are_rejected_before_any_launch():
     # an empty problem is fine and launches nothing
     cabi.sort_gaussian(0, 64, 64, 16, 16, 0, 0, 0, 0, 0, 0)
     cabi.preprocess(0, 0, 0, 0, 0, 64, 64, 16, 16, cam[0], cam[1], 1.0, 1.0, 100.0, 0.01, 0, 0, 0, 0, 0, 256)
+
+
+def test_colour_sums_switch_round_trips_and_rejects_unknown_modes():
+    prev = cabi.set_colour_sums(cabi.COLOUR_SUMS_FP32)
+    try:
+        assert prev in (cabi.COLOUR_SUMS_MATRIX_F16, cabi.COLOUR_SUMS_FP32)
+        assert cabi.set_colour_sums(cabi.COLOUR_SUMS_MATRIX_F16) == cabi.COLOUR_SUMS_FP32
+        with pytest.raises(RuntimeError, match="unknown"):
+            cabi.set_colour_sums(7)
+        assert cabi.set_colour_sums(cabi.COLOUR_SUMS_MATRIX_F16) == cabi.COLOUR_SUMS_MATRIX_F16
+    finally:
+        cabi.set_colour_sums(prev)

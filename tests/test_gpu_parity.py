@@ -584,6 +584,43 @@ def test_blend_colours_up_to_the_f16_range(oracle):
     assert np.all(np.abs(got - ref) <= 2.0 ** -10 * np.abs(ref) + 1e-4)
 
 
+@pytest.mark.parametrize("W,H,block", [(1280, 720, (16, 16)), (5120, 2880, (16, 16)), (1000, 600, (32, 16)), (1000, 600, (32, 32))])
+def test_fp32_colour_sums_mode(oracle, W, H, block):
+    """fgs_set_colour_sums(FGS_COLOUR_SUMS_FP32): the colour sums by fp32 multiply-add.  The image is
+    then as close to the oracle as the exponent's evaluation order allows, far inside the f16 bound
+    of the default mode, on the kernel of small frames, the one of large frames and both wide tiles."""
+    import gpu_pipeline as gp
+    from flashgs_amd import cabi
+    sc = scenes.config0(n=60_000)
+    cam = sc.cameras[0]
+    scale = H / cam.height
+    cam.width, cam.height = W, H
+    cam.focal_x *= scale
+    cam.focal_y *= scale
+    bg = np.array([0.3, 0.5, 0.7], np.float32)
+    ref = _oracle_frame(oracle, sc, cam, 1 << 22, block=block, bg=bg)
+    K = ref["K"]
+    got = gp.preprocess(gp.SceneOnDevice(sc), cam, 1 << 22, block=block)
+    assert got["num_rendered"] == K
+    ks, vs = gp.sort(K, W, H, got["keys"], got["values"], block)
+    images = {}
+    prev = cabi.set_colour_sums(cabi.COLOUR_SUMS_FP32)
+    try:
+        for mode in (cabi.COLOUR_SUMS_FP32, cabi.COLOUR_SUMS_MATRIX_F16):
+            cabi.set_colour_sums(mode)
+            assert ("true" if mode == cabi.COLOUR_SUMS_FP32 else "false") in cabi.blend_kernel_name(block[0], block[1], W, H)
+            _, u8, f32 = gp.render(K, W, H, got["points_xy"], got["rgb_depth"], got["conic_opacity"], ks, vs, bg, block)
+            images[mode] = (u8.cpu().numpy(), f32.cpu().numpy())
+    finally:
+        cabi.set_colour_sums(prev)
+    err32 = np.abs(images[cabi.COLOUR_SUMS_FP32][1] - ref["f32"])
+    err16 = np.abs(images[cabi.COLOUR_SUMS_MATRIX_F16][1] - ref["f32"])
+    assert err32.max() <= 2e-4, "fp32 colour sums: max abs image error %g" % err32.max()
+    assert err16.max() <= IMG_MAX_ABS and err32.mean() < err16.mean()
+    d8 = np.abs(images[cabi.COLOUR_SUMS_FP32][0].astype(np.int16) - ref["u8"].astype(np.int16))
+    assert d8.max() <= 1 and (d8 > 0).mean() < 0.005
+
+
 def test_ranges_kernel_against_searchsorted():
     import gpu_pipeline as gp
     import torch
