@@ -314,13 +314,6 @@ def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops):
                                  stages_ms_mean={k: round(v, 4) for k, v in traj_stage.items()})
     if with_ops:
         rep["ops_surface_ms_per_frame"], rep["ops_surface_image_identical"] = ops_surface_ms(torch, np, fr, steps)
-        # the same frame with the colour sums by fp32 multiply-add instead of the matrix unit (fgs_set_colour_sums)
-        prev = cabi.set_colour_sums(cabi.COLOUR_SUMS_FP32)
-        try:
-            ms32, stage32, _, _ = fr.timed(fr.cams[:1], max(5, steps // 2), 2, False)
-        finally:
-            cabi.set_colour_sums(prev)
-        rep["fp32_colour_sums"] = dict(ms_per_frame=round(ms32, 4), blend_ms=round(stage32["blend"], 4))
     return rep, fr
 
 
@@ -350,6 +343,14 @@ def main():
     with_cpu = not args.no_cpu_baseline
 
     head, fr = run_config(mods, args.config, size, args.steps, args.warmup, args.cpu_reps, with_cpu, True)
+    if not args.headline_only:
+        # the same frame with the colour sums by fp32 multiply-add instead of the matrix unit (fgs_set_colour_sums)
+        prev = cabi.set_colour_sums(cabi.COLOUR_SUMS_FP32)
+        try:
+            ms32, stage32, _, _ = fr.timed(fr.cams[:1], max(5, args.steps // 2), 2, False)
+        finally:
+            cabi.set_colour_sums(prev)
+        head["fp32_colour_sums"] = dict(ms_per_frame=round(ms32, 4), blend_ms=round(stage32["blend"], 4))
     if args.copy_calibration:
         src = torch.ones(64 << 20, device=dev, dtype=torch.float32)      # 256 MiB read + 256 MiB written
         dst = torch.empty_like(src)
