@@ -10,7 +10,9 @@
 // batch are already in flight; the wave then walks the batch, every lane reading the table
 // entries of its own columns and rows.  After every second Gaussian one ballot tests whether all
 // pixels of the tile have T < 1e-4, which is the reference's stop rule (render.cu:394-408).  A
-// workgroup is a single wave, so no workgroup barrier is needed anywhere.
+// workgroup is a single wave, so no workgroup barrier is needed anywhere.  The colour sums go
+// through the matrix unit four Gaussians at a time (f16 operands, fp32 accumulation) or, on
+// request (fgs_set_colour_sums), through fp32 multiply-adds; every kernel exists in both forms.
 #include "fgs_internal.h"
 
 #include <atomic>
@@ -200,7 +202,7 @@ constexpr int kGroups = kBatch / 4;
 // products and sums are fp32: the colour of a pixel differs from the all-fp32 sum by at most
 // 2^-10 of itself.  The weights are scaled by 2^14 (added to the exponent when it is tabulated,
 // taken out again with the result), which keeps them in f16's normal range down to 4e-9.
-// T itself never leaves fp32.
+// T itself never leaves fp32.  The template parameter kFp32 of the walk selects the other form.
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float float2_t __attribute__((ext_vector_type(2)));
