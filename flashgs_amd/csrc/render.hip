@@ -119,7 +119,7 @@ __global__ __launch_bounds__(1024) void tile_order_kernel(const int2* __restrict
 // render.cu:557): the pair that opens tile c clears the tiles between its predecessor's tile and
 // c, the first pair those before it and the last pair those behind it.  A run of up to 4 tiles is
 // cleared by the thread that found it, a longer one by its whole wave.
-constexpr int kRangesPerThread = 8;
+constexpr int kRangesPerThread = 4;
 
 __global__ __launch_bounds__(256) void tile_ranges_kernel(int L, const uint64_t* __restrict__ keys,
                                                           int2* __restrict__ ranges, uint32_t num_tiles)
