@@ -722,13 +722,19 @@ def _sort_case(tile, depth_bits, W, H, junk=None, seed=0):
     assert np.array_equal(gp.u32(vs)[:n], vals[order])
 
 
+@pytest.mark.parametrize("dense", [False, True])
 @pytest.mark.parametrize("seg", [1500, 3000, 5000, 8000, 8192, 8193, 40000])
-def test_sort_segment_size_classes(seg):
+def test_sort_segment_size_classes(seg, dense):
     """Tiles holding 1500 ... 40000 pairs: every size class of the per-tile depth sort, with many
-    equal depths and with depths that agree in whole bytes (skipped passes)."""
+    equal depths and with depths that agree in whole bytes (skipped passes); on a frame of many
+    tiles with few pairs and on one of 16 tiles with thousands of pairs each."""
     rng = np.random.default_rng(seg)
-    W, H = 1920, 1080
-    tile = np.repeat(np.array([5, 6, 4000, 8159], np.uint32), [seg, 7, seg // 2, seg])
+    if dense:
+        W, H = 64, 64
+        tile = np.repeat(np.array([5, 6, 9, 15, 1], np.uint32), [seg, 7, seg // 2, seg, 20000])
+    else:
+        W, H = 1920, 1080
+        tile = np.repeat(np.array([5, 6, 4000, 8159], np.uint32), [seg, 7, seg // 2, seg])
     rng.shuffle(tile)
     depth = rng.uniform(1.0, 1.9, tile.size).astype(np.float32)      # same exponent: top byte constant
     depth[::3] = np.float32(1.5)
