@@ -10,7 +10,9 @@ and every work buffer are allocated once, outside the timed region.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..4] [--no-cpu-baseline] [--headline-only]
 
 Prints one JSON line.  ``value`` is frames per second of the whole frame on the headline workload
-(``--config``, default the 4K / 3M one); ``roofline`` describes its dominant kernel (the blend),
+(``--config``, default the 4K / 3M one) with the library's default arithmetic, fp32 throughout as
+the reference computes; the same frame with the opt-in colour sums on the matrix unit (f16
+operands) is reported beside it as ``fast_mode_*``.  ``roofline`` describes the dominant kernel (the blend),
 ``stages`` every stage with its algorithmic bytes against the 8 TB/s HBM peak, ``cpu_baseline`` the
 same frame computed by the multithreaded CPU oracle on this machine's host cores,
 ``ops_surface_ms_per_frame`` the same frame through ``flash_gaussian_splatting.ops`` the way
@@ -31,10 +33,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3         # MI355X fp32 vector, published (packed FMA)
-LANE_SLOTS_PER_S = 256 * 4 * 16 * 2.4e9   # VALU issue slots per second without packed math
 FLOP_PER_EVAL = 19               # render.cu:40-52: 2 sub, 6 mul + 3 add, 1 mul, 3 FMA, 1 sub
-SLOTS_PER_EVAL = 17              # 13 VALU with FMA contraction + a quarter-rate exp2 (the reference formulation)
-CAPACITY = {0: 1 << 20, 1: 1 << 22, 2: 1 << 24, 3: 1 << 25, 4: 1 << 25}
+EXEC_SLOTS_PER_EVAL = 9          # what the fp32 blend kernel issues: 2 for the exponent from its tables, exp2 at half
+                                 # rate = 2, alpha*T, T -= , 3 colour FMAs
+ATTAINED_FMA_LANE_OPS = 38.05e12 # v_fma_f32 lane-operations/s measured on this part without packed math (bench.py --calibrate)
+CAPACITY = {0: 1 << 20, 1: 1 << 22, 2: 1 << 24, 3: 1 << 25, 4: 1 << 25, 5: 1 << 27}
+FAST_MODE_DTYPE = "f32 (colour sums: f16 operands on the matrix unit, fp32 products and sums)"
 
 
 def parse():
@@ -42,7 +46,9 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", type=int, default=2, help="index into BASELINE.json configs (default: the 4K / 3M headline)")
+    ap.add_argument("--config", type=int, default=2,
+                    help="index into BASELINE.json configs (default: the 4K / 3M headline); 5 = the 8K scene with every "
+                         "splat five times as large (more than 100M pairs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-reps", type=int, default=3)
     ap.add_argument("--headline-only", action="store_true", help="skip the other configurations (field \"configs\")")
@@ -144,10 +150,12 @@ def profiled_traffic(workload, kernel):
 class Frame:
     """One configuration resident on the GPU with every buffer a frame needs."""
 
-    def __init__(self, torch, np, cabi, scenes, config, size=None):
+    def __init__(self, torch, np, cabi, scenes, config, size=None, base=None):
         kw = {}
         if size:
             kw["width"], kw["height"] = size
+        if base is not None:
+            kw["base"] = base
         self.torch, self.np, self.cabi = torch, np, cabi
         self.sc = scenes.make(config, **kw)
         self.cams = self.sc.cameras
@@ -182,7 +190,8 @@ class Frame:
             "position", "shs", "opacity", "cov3d", "points_xy", "rgb_depth", "conic_opacity", "keys_u", "vals_u",
             "keys_s", "vals_s", "sort_space", "ranges", "curr_offset", "out_color")}
 
-    def frame(self, c, ev=None):
+    def frame(self, c, ev=None, flags=None):
+        """One frame; `flags` (cabi.BLEND_*) chooses the blend's colour-sum mode for this call, None = the library default."""
         cabi, P, W, H, st = self.cabi, self.P, self.W, self.H, self.stream
         if ev: ev[0].record()
         self.curr_offset.zero_()
@@ -200,15 +209,15 @@ class Frame:
         cabi.tile_ranges(16, 16, K, W, H, P["keys_s"], P["ranges"], st)
         if ev: ev[4].record()
         cabi.blend(16, 16, W, H, P["points_xy"], P["rgb_depth"], P["conic_opacity"], P["vals_s"], P["ranges"], self.bg,
-                   P["out_color"], None, st)
+                   P["out_color"], None, st, flags=flags)
         if ev: ev[5].record()
         return K
 
-    def timed(self, cams, steps, warmup, per_frame_sync):
+    def timed(self, cams, steps, warmup, per_frame_sync, flags=None):
         """steps frames over `cams` in turn: (ms per step, per-stage mean ms, per-frame ms or [], pair count of the first)."""
         torch = self.torch
         for i in range(warmup):
-            self.frame(cams[i % len(cams)])
+            self.frame(cams[i % len(cams)], flags=flags)
         torch.cuda.synchronize()
         events = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(steps)]
         frame_ms, Ks = [], []
@@ -216,7 +225,7 @@ class Frame:
         t_start = time.perf_counter()
         for i in range(steps):
             t0 = time.perf_counter()
-            Ks.append(self.frame(cams[i % len(cams)], events[i]))
+            Ks.append(self.frame(cams[i % len(cams)], events[i], flags))
             if per_frame_sync:            # per-frame latency only matters for the trajectory workload
                 torch.cuda.synchronize()
                 frame_ms.append((time.perf_counter() - t0) * 1e3)
@@ -250,20 +259,23 @@ def stage_report(fr, stage_ms, K, counts, walked):
     stages["readback"] = dict(ms=round(stage_ms["readback"], 4), bound="host latency (4-byte read + sync)")
 
     blend_ms = stage_ms["blend"]
-    kernel = fr.cabi.blend_kernel_name(16, 16, W, H)
+    kernel = fr.cabi.blend_kernel_name(16, 16, W, H)        # of the library default, which is what was timed
     traffic, source = profiled_traffic(fr.sc.name, kernel)
     roofline = dict(kernel=kernel, bound="valu", achieved=None, peak=FP32_PEAK_TFLOPS, unit="TFLOP/s", frac=None,
                     traffic=traffic, traffic_source=source, launch_ms=round(blend_ms, 4))
     stages["blend"] = dict(ms=round(blend_ms, 4), bound="valu", kernel=kernel)
     if walked is not None:
         evals = 256 * walked
+        # reference-equivalent work: the 19 flop of render.cu:40-52 per pixel-Gaussian evaluation over the
+        # published fp32 vector peak (which counts packed FMA; this library issues none)
         tflops = FLOP_PER_EVAL * evals / (blend_ms * 1e-3) / 1e12
+        # executed work: the kernel's own 9 issue slots per evaluation over the v_fma_f32 rate this part attains
+        floor_ms = EXEC_SLOTS_PER_EVAL * evals / ATTAINED_FMA_LANE_OPS * 1e3
         roofline.update(achieved=round(tflops, 2), frac=round(tflops / FP32_PEAK_TFLOPS, 4),
+                        achieved_is="reference-equivalent flop (19 per evaluation, render.cu:40-52) per second",
                         evaluations=int(evals), flop_per_evaluation=FLOP_PER_EVAL,
-                        # VALU issue slots the reference's formula would take (13 + 4 for exp2 per evaluation)
-                        # over the slots the chip has in that time: above 1, because the kernel gets the
-                        # exponent from tabulated parts (8.1 VALU instructions per evaluation measured)
-                        reference_formula_issue_slot_frac=round(SLOTS_PER_EVAL * evals / (blend_ms * 1e-3) / LANE_SLOTS_PER_S, 4),
+                        executed_issue_slots_per_evaluation=EXEC_SLOTS_PER_EVAL,
+                        issue_bound_ms=round(floor_ms, 4), frac_of_attained_issue_rate=round(floor_ms / blend_ms, 4),
                         hbm_bytes=int(8 * tiles + 44 * walked + 3 * W * H))
         stages["blend"].update(achieved_TFLOPs=roofline["achieved"], frac=roofline["frac"])
     return stages, roofline
@@ -291,17 +303,22 @@ def ops_surface_ms(torch, np, fr, steps):
     return round(ms, 4), same
 
 
-def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops):
+def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops, base=None):
     torch, np, cabi, scenes = mods
-    fr = Frame(torch, np, cabi, scenes, config, size)
+    fr = Frame(torch, np, cabi, scenes, config, size, base)
     ms_per_step, stage_ms, _, K = fr.timed(fr.cams[:1], steps, warmup, False)
+    # the same frame with the opt-in colour sums on the matrix unit, chosen per call
+    fast_ms, fast_stage, _, _ = fr.timed(fr.cams[:1], max(5, steps // 2), 2, False, flags=cabi.BLEND_MATRIX_F16)
     cpu, counts, walked = (None, None, None)
     if with_cpu:
         cpu, counts, walked = cpu_baseline(fr.sc, fr.cams[0], fr.capacity, cpu_reps)
     stages, roofline = stage_report(fr, stage_ms, K, counts, walked)
     rep = dict(workload=fr.sc.name, gaussians=fr.n, width=fr.W, height=fr.H, pairs=int(K), poses=len(fr.cams),
-               ms_per_frame=round(ms_per_step, 4), fps=round(1000.0 / ms_per_step, 2), stages=stages, roofline=roofline,
-               cpu_baseline=cpu)
+               ms_per_frame=round(ms_per_step, 4), fps=round(1000.0 / ms_per_step, 2), dtype="f32", stages=stages,
+               roofline=roofline, cpu_baseline=cpu,
+               fast_mode=dict(dtype=FAST_MODE_DTYPE, ms_per_frame=round(fast_ms, 4), fps=round(1000.0 / fast_ms, 2),
+                              blend_ms=round(fast_stage["blend"], 4),
+                              kernel=cabi.blend_kernel_name(16, 16, fr.W, fr.H, cabi.BLEND_MATRIX_F16)))
     if counts is not None:
         rep.update(n_pass=counts["n_pass"], visible=counts["visible"], walked=int(walked))
     if len(fr.cams) > 1:
@@ -343,14 +360,6 @@ def main():
     with_cpu = not args.no_cpu_baseline
 
     head, fr = run_config(mods, args.config, size, args.steps, args.warmup, args.cpu_reps, with_cpu, True)
-    if not args.headline_only:
-        # the same frame with the colour sums by fp32 multiply-add instead of the matrix unit (fgs_set_colour_sums)
-        prev = cabi.set_colour_sums(cabi.COLOUR_SUMS_FP32)
-        try:
-            ms32, stage32, _, _ = fr.timed(fr.cams[:1], max(5, args.steps // 2), 2, False)
-        finally:
-            cabi.set_colour_sums(prev)
-        head["fp32_colour_sums"] = dict(ms_per_frame=round(ms32, 4), blend_ms=round(stage32["blend"], 4))
     if args.copy_calibration:
         src = torch.ones(64 << 20, device=dev, dtype=torch.float32)      # 256 MiB read + 256 MiB written
         dst = torch.empty_like(src)
@@ -363,14 +372,18 @@ def main():
         "value": head["fps"], "unit": "frames/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": head["ms_per_frame"], "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32",
-        "dtype_note": "fp32 throughout (ndc2Pix fp64 as the reference); the blend's colour sums take f16 operands "
-                      "(weights alpha*T, colours) with fp32 products and accumulation, within 2^-10 of a pixel's colour",
+        "vs_baseline": None, "dtype": head["dtype"],
+        "dtype_note": "every stage in fp32 as the reference (ndc2Pix in fp64 as its literals make it); the timed blend "
+                      "kernel is the one named in roofline.kernel",
         "data": "synthetic",
         "config": {"workload": head["workload"], "gaussians": head["gaussians"], "width": head["width"], "height": head["height"],
-                   "tile": "16x16", "sh_degree": 3, "pairs": head["pairs"], "poses": head["poses"]},
+                   "tile": "16x16", "sh_degree": 3, "pairs": head["pairs"], "poses": head["poses"],
+                   "stages_ms": {k: v["ms"] for k, v in head["stages"].items()},
+                   "fast_mode": head["fast_mode"]},
         "target_fps": 400 if args.config == 2 else None,
-        "fp32_colour_sums": head.get("fp32_colour_sums"),
+        "fast_mode_ms_per_frame": head["fast_mode"]["ms_per_frame"],
+        "fast_mode_fps": head["fast_mode"]["fps"],
+        "fast_mode_dtype": FAST_MODE_DTYPE,
         "stages": head["stages"],
         "roofline": head["roofline"],
         "cpu_baseline": head["cpu_baseline"],
@@ -391,11 +404,14 @@ def main():
 
     if not args.headline_only:
         others = {}
-        for config, sz in ((0, None), (1, None), (2, None), (3, None), (4, None), (4, (3840, 2160))):
+        big = None          # the 8M scene, generated once for the 8K configuration and its dense variant
+        for config, sz in ((0, None), (1, None), (2, None), (3, None), (5, None), (4, None), (4, (3840, 2160))):
             if config == args.config and sz == size:
                 continue
-            rep, fr_o = run_config(mods, config, sz, args.other_steps, min(args.warmup, 3), 1, with_cpu, False)
+            rep, fr_o = run_config(mods, config, sz, args.other_steps, min(args.warmup, 3), 1, with_cpu, False,
+                                   base=big if config == 5 else None)
             others[rep["workload"]] = rep
+            big = fr_o.sc if config == 3 else (None if config == 5 else big)
             del fr_o
             torch.cuda.empty_cache()
         result["configs"] = others

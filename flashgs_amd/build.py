@@ -4,8 +4,10 @@
 Everything is compiled for gfx950 only and lands in-tree (``flashgs_amd/lib/`` and the
 repository root), so a copy of the tree carries the binaries with it.
 
-    python -m flashgs_amd.build            # both
-    python -m flashgs_amd.build --lib      # only the C-ABI library
+    python -m flashgs_amd.build              # both
+    python -m flashgs_amd.build --lib        # only the C-ABI library
+    python -m flashgs_amd.build --asan-host  # flashgs_amd/lib/asan/host_checks: the library's host code and the .ply
+                                             # reader under the address and undefined-behaviour sanitizers (CPU only)
 """
 import os
 import subprocess
@@ -52,6 +54,30 @@ def build_lib():
     return LIB_PATH
 
 
+ASAN_DIR = os.path.join(LIB_DIR, "asan")
+ASAN_CHECKS = os.path.join(ASAN_DIR, "host_checks")
+# sanitizers on the host code only: each -fsanitize= directly behind -Xarch_host
+ASAN_HOST = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+             "-Xarch_host", "-fno-sanitize-recover=undefined", "-g", "-fno-omit-frame-pointer"]
+
+
+def build_asan_host():
+    """host_checks.cpp linked with the library's own translation units, host code instrumented.
+    Run it as ``ASAN_OPTIONS=detect_leaks=0 flashgs_amd/lib/asan/host_checks`` (the HIP runtime keeps
+    allocations of its own until the process ends); it launches nothing and needs no GPU."""
+    os.makedirs(ASAN_DIR, exist_ok=True)
+    objs = []
+    for src, extra in SOURCES.items():
+        obj = os.path.join(ASAN_DIR, src.replace(".hip", ".o"))
+        _run([HIPCC] + HIP_FLAGS + ASAN_HOST + extra + ["-c", os.path.join(CSRC, src), "-o", obj])
+        objs.append(obj)
+    main = os.path.join(ASAN_DIR, "host_checks.o")
+    _run([HIPCC, "-x", "hip"] + HIP_FLAGS + ASAN_HOST + ["-I", os.path.join(ROOT, "include"), "-c",
+                                                        os.path.join(CSRC, "host_checks.cpp"), "-o", main])
+    _run([HIPCC, "--offload-arch=gfx950", "-fno-gpu-sanitize", "-fsanitize=address", "-fsanitize=undefined", "-o", ASAN_CHECKS, main] + objs)
+    return ASAN_CHECKS
+
+
 def ext_path():
     suffix = sysconfig.get_config_var("EXT_SUFFIX")
     return os.path.join(ROOT, "flash_gaussian_splatting" + suffix)
@@ -91,5 +117,7 @@ def build_all():
 if __name__ == "__main__":
     if "--lib" in sys.argv:
         build_lib()
+    elif "--asan-host" in sys.argv:
+        build_asan_host()
     else:
         build_all()

@@ -30,9 +30,12 @@ SIGNATURES = {
     "fgs_render_f32": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 9 + [C.c_void_p]),
     "fgs_tile_ranges": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 3),
     "fgs_blend": (C.c_int, [C.c_int] * 4 + [C.c_void_p] * 9),
-    "fgs_blend_kernel_name": (C.c_char_p, [C.c_int] * 4),
+    "fgs_render_ex": (C.c_int, [C.c_int] * 5 + [C.c_void_p] * 9 + [C.c_int, C.c_void_p]),
+    "fgs_blend_ex": (C.c_int, [C.c_int] * 4 + [C.c_void_p] * 8 + [C.c_int, C.c_void_p]),
+    "fgs_blend_kernel_name": (C.c_char_p, [C.c_int] * 5),
     "fgs_camera_matrices": (None, [C.c_void_p] * 2 + [C.c_int] * 2 + [C.c_float] * 4 + [C.c_void_p] * 2),
     "fgs_set_scan_spin_limit": (C.c_uint, [C.c_uint]),
+    "fgs_reset_scan": (C.c_int, [C.c_void_p]),
     "fgs_set_colour_sums": (C.c_int, [C.c_int]),
     "fgs_last_error": (C.c_char_p, []),
     "fgs_abi_version": (C.c_int, []),
@@ -95,11 +98,12 @@ def preprocess(P, positions, shs, opacities, cov3ds, width, height, block_x, blo
 
 
 COLOUR_SUMS_MATRIX_F16, COLOUR_SUMS_FP32 = 0, 1
+BLEND_DEFAULT, BLEND_FP32, BLEND_MATRIX_F16 = 0, 1, 2       # the flags of render_f32 / blend / blend_kernel_name
 
 
 def set_colour_sums(mode):
-    """How later blends form their colour sums (matrix unit with f16 operands, or fp32 multiply-add);
-    returns the previous mode."""
+    """The process default of how blends form their colour sums (fp32 multiply-add, or the matrix
+    unit with f16 operands); returns the previous default."""
     prev = int(load().fgs_set_colour_sums(int(mode)))
     if prev < 0:
         raise RuntimeError("fgs_set_colour_sums failed: %s" % last_error())
@@ -109,6 +113,11 @@ def set_colour_sums(mode):
 def set_scan_spin_limit(polls):
     """Polls after which a wait inside the preprocess launch gives up; returns the previous value."""
     return int(load().fgs_set_scan_spin_limit(polls))
+
+
+def reset_scan(stream=0):
+    """Clears the scan status of preprocess on `stream` (the way back after a negative pair count)."""
+    _check(load().fgs_reset_scan(stream), "fgs_reset_scan")
 
 
 def get_sort_buffer_size(num_rendered):
@@ -134,16 +143,22 @@ def render(block_x, block_y, num_rendered, width, height, points_xy, rgb_depth, 
 
 
 def render_f32(block_x, block_y, num_rendered, width, height, points_xy, rgb_depth, conic_opacity,
-               keys_sorted, values_sorted, ranges, bg_color, out_u8, out_f32, stream=0):
+               keys_sorted, values_sorted, ranges, bg_color, out_u8, out_f32, stream=0, flags=None):
+    """fgs_render_f32, or fgs_render_ex when `flags` (BLEND_*) is given."""
     bg = _host_f32(bg_color, 3)
-    rc = load().fgs_render_f32(block_x, block_y, num_rendered, width, height, points_xy, rgb_depth, conic_opacity,
-                               keys_sorted, values_sorted, ranges, bg.ctypes.data, out_u8, out_f32, stream)
-    _check(rc, "fgs_render_f32")
+    if flags is None:
+        rc = load().fgs_render_f32(block_x, block_y, num_rendered, width, height, points_xy, rgb_depth, conic_opacity,
+                                   keys_sorted, values_sorted, ranges, bg.ctypes.data, out_u8, out_f32, stream)
+        _check(rc, "fgs_render_f32")
+    else:
+        rc = load().fgs_render_ex(block_x, block_y, num_rendered, width, height, points_xy, rgb_depth, conic_opacity,
+                                  keys_sorted, values_sorted, ranges, bg.ctypes.data, out_u8, out_f32, int(flags), stream)
+        _check(rc, "fgs_render_ex")
 
 
-def blend_kernel_name(block_x, block_y, width, height):
+def blend_kernel_name(block_x, block_y, width, height, flags=BLEND_DEFAULT):
     """The kernel(s) a blend of this tile and frame size launches on the current device."""
-    return load().fgs_blend_kernel_name(block_x, block_y, width, height).decode()
+    return load().fgs_blend_kernel_name(block_x, block_y, width, height, int(flags)).decode()
 
 
 def tile_ranges(block_x, block_y, num_rendered, width, height, keys_sorted, ranges, stream=0):
@@ -152,7 +167,12 @@ def tile_ranges(block_x, block_y, num_rendered, width, height, keys_sorted, rang
 
 
 def blend(block_x, block_y, width, height, points_xy, rgb_depth, conic_opacity, values_sorted, ranges, bg_color,
-          out_u8, out_f32, stream=0):
+          out_u8, out_f32, stream=0, flags=None):
+    """fgs_blend, or fgs_blend_ex when `flags` (BLEND_*) is given."""
     bg = _host_f32(bg_color, 3)
-    _check(load().fgs_blend(block_x, block_y, width, height, points_xy, rgb_depth, conic_opacity, values_sorted,
-                            ranges, bg.ctypes.data, out_u8, out_f32, stream), "fgs_blend")
+    if flags is None:
+        _check(load().fgs_blend(block_x, block_y, width, height, points_xy, rgb_depth, conic_opacity, values_sorted,
+                                ranges, bg.ctypes.data, out_u8, out_f32, stream), "fgs_blend")
+    else:
+        _check(load().fgs_blend_ex(block_x, block_y, width, height, points_xy, rgb_depth, conic_opacity, values_sorted,
+                                   ranges, bg.ctypes.data, out_u8, out_f32, int(flags), stream), "fgs_blend_ex")

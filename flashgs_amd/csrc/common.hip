@@ -29,4 +29,4 @@ int check_hip(hipError_t st, const char* what)
 
 extern "C" const char* fgs_last_error(void) { return fgs::g_last_error; }
 
-extern "C" int fgs_abi_version(void) { return 1; }
+extern "C" int fgs_abi_version(void) { return FGS_ABI_VERSION; }

@@ -26,6 +26,7 @@
 #include <map>
 #include <mutex>
 #include <utility>
+#include <vector>
 
 namespace fgs {
 namespace {
@@ -342,7 +343,18 @@ __device__ __forceinline__ void sh_to_rgb(const float* __restrict__ sh, float px
 // workgroup that gave up on its offset (or found it poisoned) writes its keys from slot 0 and
 // lowers *curr_offset to INT_MIN, and the scanner's own final write of the total is a
 // compare-and-swap against the starting value, so INT_MIN stays whichever comes first.
+//
+// A scanner that gives up does so before it has seen every count, i.e. possibly before every
+// workgroup of the launch has been dispatched, so it must not hand the other generation on: a
+// workgroup dispatched after a flip would take the wrong generation, clear the arrays the others
+// publish in and leave words behind that the next launch would take for its own.  Instead it
+// sets the "aborted" bit of the control word and leaves the generation alone.  The bit is sticky:
+// every workgroup that finds it - the rest of this launch and every later launch on these scan
+// words - does nothing but lower *curr_offset to INT_MIN, until the host clears the words
+// (fgs_reset_scan), which is the one way back to a state in which all status words are zero.
 constexpr int kControlWords = 8;          // control word + padding in front of the arrays
+constexpr uint64_t kControlGeneration = 1;  // control word: which generation this launch works in ...
+constexpr uint64_t kControlAborted = 2;     // ... and whether a scanner on these words has given up
 constexpr uint64_t kStateCount = 1;       // key count of one workgroup
 constexpr uint64_t kStateOffset = 2;      // number of keys in front of a workgroup
 constexpr uint64_t kStatePoison = 3;      // the offset could not be computed
@@ -370,7 +382,7 @@ __device__ __forceinline__ uint64_t peek(const uint64_t* slot)
 // frame (0.203 ms for the launch against 0.207 with 256, 0.219 with 512 and 0.256 with 1024).
 constexpr int kScanPerLane = 2;
 
-__device__ __forceinline__ void scan_counts(const uint64_t* counts, uint64_t* offsets, int num_blocks,
+__device__ __forceinline__ bool scan_counts(const uint64_t* counts, uint64_t* offsets, int num_blocks,
                                             int* curr_offset, unsigned spin_limit)
 {
     const int lane = lane_id();
@@ -417,6 +429,7 @@ __device__ __forceinline__ void scan_counts(const uint64_t* counts, uint64_t* of
     } else if (lane == 0) {
         atomicCAS(curr_offset, (int)start, (int)running);
     }
+    return gave_up;
 }
 
 // Executed by one lane of a workgroup: the number of keys in front of the workgroup, once the
@@ -468,15 +481,25 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     __shared__ int s_huge_spans[kHugeCap];                      // 1: the tiles that pass are found from column and row spans
     __shared__ int s_nhuge;
     __shared__ int s_centre[2];                                 // column and row of a listed rectangle that hold its centre
+    __shared__ uint32_t s_control;
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    if (tid == 0) s_nhuge = 0;
+    if (tid == 0) {
+        s_nhuge = 0;
+        s_control = (uint32_t)peek(scan_words);     // one read per workgroup: all its threads must agree on it
+    }
     __syncthreads();
+    const uint32_t control = s_control;
+    if (control & kControlAborted) {
+        // a scanner on these words gave up (in this launch or an earlier one): touch nothing
+        if (tid == 0) atomicMin(curr_offset, kIntMin);
+        return;
+    }
 
     // this launch's generation of the scan words; the other one is cleared for the launch that follows
-    const uint32_t which = (uint32_t)peek(scan_words) & 1u;
+    const uint32_t which = control & (uint32_t)kControlGeneration;
     uint64_t* const counts = scan_words + kControlWords + (size_t)which * 2 * status_capacity;
     uint64_t* const offsets = counts + status_capacity;
     {
@@ -489,9 +512,11 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     // later one waits for its offset (and every wait is bounded in any case).
     if (blockIdx.x == 0) {
         if (wave == 0) {
-            scan_counts(counts, offsets, num_blocks, curr_offset, spin_limit);
-            // every workgroup has read the control word by now: hand the other generation to the next launch
-            if (lane == 0) publish(scan_words, (uint64_t)(which ^ 1u));
+            const bool gave_up = scan_counts(counts, offsets, num_blocks, curr_offset, spin_limit);
+            // Read every count: every workgroup has read the control word by now, so the other
+            // generation can be handed to the next launch.  Gave up: workgroups may still be
+            // dispatched; the generation stays and the words are marked unusable.
+            if (lane == 0) publish(scan_words, gave_up ? (uint64_t)which | kControlAborted : (uint64_t)(which ^ 1u));
         }
         return;
     }
@@ -556,8 +581,9 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
                 // preprocess.cu:90-100
                 rminx = min(cam.gx, max(0, to_int_sat((cx - (float)ext_x) / (float)cam.bx)));
                 rminy = min(cam.gy, max(0, to_int_sat((cy - (float)ext_y) / (float)cam.by)));
-                int rmaxx = min(cam.gx, max(0, to_int_sat((cx + (float)ext_x) / (float)cam.bx) + 1));
-                int rmaxy = min(cam.gy, max(0, to_int_sat((cy + (float)ext_y) / (float)cam.by) + 1));
+                // (the "+ 1" wraps at INT_MAX, as the integer add of the reference's device does: written out, not left to overflow)
+                int rmaxx = min(cam.gx, max(0, (int)((uint32_t)to_int_sat((cx + (float)ext_x) / (float)cam.bx) + 1u)));
+                int rmaxy = min(cam.gy, max(0, (int)((uint32_t)to_int_sat((cy + (float)ext_y) / (float)cam.by) + 1u)));
                 rw = rmaxx - rminx;
                 rh = rmaxy - rminy;
                 cand = rw * rh > 0;
@@ -937,16 +963,37 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
 //
 // Launches on one stream follow each other, so they can share one set of scan words; launches on
 // different streams of a device may overlap in time and get a set each.  A set is allocated on
-// the first call on its stream and grown when a larger P arrives (the only times a call
-// synchronises), and lives until the process ends.
+// the first call on its stream; when a larger P arrives a larger set is allocated and the stream
+// uses that one from then on.  No set is ever freed: a HIP graph captured on the stream holds the
+// address of the set its launch used in its kernel node, and replaying it after a free would make
+// every workgroup read and write freed memory.  A retired set costs 32 bytes per 256 Gaussians of
+// the P it was sized for and keeps serving the graphs that know it (its own control word and
+// generations stay consistent: launches on one stream, replayed or not, follow each other).
 
 struct Scratch {
     uint64_t* words = nullptr;      // control word (+ padding), then two generations of (counts, offsets)
     size_t capacity = 0;            // workgroups each of the four arrays holds
 };
 
+__global__ __launch_bounds__(256) void clear_words_kernel(uint64_t* words, size_t n)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) words[i] = 0;
+}
+
+// Zeroes n words on the stream with a kernel (not a memset node, so that it may be captured).
+int clear_words(uint64_t* words, size_t n, hipStream_t stream)
+{
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL(clear_words_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, words, n);
+    return check_hip(hipGetLastError(), "clear_words_kernel launch");
+}
+
 constexpr int kMaxDevices = 64;
 std::map<StreamKey, Scratch> g_scratch;
+std::vector<uint64_t*> g_retired;   // sets replaced by larger ones: kept, since captured graphs may hold their addresses
 std::mutex g_mutex;
 std::atomic<unsigned> g_spin_limit{kSpinLimit};
 
@@ -960,20 +1007,20 @@ int acquire_scratch(int device, int num_blocks, hipStream_t stream, Scratch** ou
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         if (stream) FGS_HIP_TRY(hipStreamIsCapturing(stream, &capture));
         if (capture != hipStreamCaptureStatusNone) return FGS_OK;
-        // the stream may still be reading the old arrays: drain it before the swap
-        FGS_HIP_TRY(hipStreamSynchronize(stream));
-        if (s.words) FGS_HIP_TRY(hipFree(s.words));
-        s.words = nullptr;
-        s.capacity = 0;
         size_t cap = 4096;
         while (cap < (size_t)num_blocks) cap <<= 1;
-        const size_t bytes = (kControlWords + 4 * cap) * sizeof(uint64_t);
-        if (hipMalloc((void**)&s.words, bytes) != hipSuccess) {
+        const size_t words = kControlWords + 4 * cap;
+        uint64_t* fresh = nullptr;
+        if (hipMalloc((void**)&fresh, words * sizeof(uint64_t)) != hipSuccess) {
             (void)hipGetLastError();
-            return fail(FGS_E_NOMEM, "cannot allocate %zu bytes of scan status", bytes);
+            return fail(FGS_E_NOMEM, "cannot allocate %zu bytes of scan status", words * sizeof(uint64_t));
         }
-        FGS_HIP_TRY(hipMemset(s.words, 0, bytes));
-        FGS_HIP_TRY(hipDeviceSynchronize());
+        // cleared on the stream itself, in front of the launch that uses it first; the set in use
+        // so far (if any) is left alone and alive for the launches and graphs that hold its address
+        int rc = clear_words(fresh, words, stream);
+        if (rc != FGS_OK) return rc;
+        if (s.words) g_retired.push_back(s.words);
+        s.words = fresh;
         s.capacity = cap;
     }
     *out = &s;
@@ -1130,6 +1177,26 @@ int preprocess_impl(bool allocate, const char* who, int P,
 extern "C" unsigned fgs_set_scan_spin_limit(unsigned polls)
 {
     return fgs::g_spin_limit.exchange(polls);
+}
+
+extern "C" int fgs_reset_scan(void* stream)
+{
+    using namespace fgs;
+    int device = 0;
+    FGS_HIP_TRY(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return fail(FGS_E_INVALID, "fgs_reset_scan: device %d unsupported", device);
+    hipStream_t st = (hipStream_t)stream;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    // the stream's own scan words, if it has any, and the built-in ones of the device
+    auto it = g_scratch.find(stream_key(device, st));
+    if (it != g_scratch.end() && it->second.words) {
+        int rc = clear_words(it->second.words, kControlWords + 4 * it->second.capacity, st);
+        if (rc != FGS_OK) return rc;
+    }
+    uint64_t* words = nullptr;
+    int rc = static_scratch(device, &words);
+    if (rc != FGS_OK) return rc;
+    return clear_words(words, kControlWords + 4 * (size_t)kStaticBlocks, st);
 }
 
 extern "C" int fgs_preprocess(int P,

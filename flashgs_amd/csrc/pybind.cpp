@@ -12,8 +12,6 @@
 #include <torch/extension.h>
 #include <c10/hip/HIPStream.h>
 
-#include <cmath>
-#include <cstring>
 #include <fstream>
 #include <stdexcept>
 #include <string>
@@ -21,6 +19,7 @@
 #include <vector>
 
 #include "flashgs_hip.h"
+#include "ply_reader.h"
 
 namespace {
 
@@ -185,87 +184,36 @@ void render(int num_rendered, int width, int height,
 
 // ---- loadPly (pybind.cpp:12-120) --------------------------------------------------------------------
 //
-// Reads the binary little-endian .ply that 3DGS training writes: after the text header, one
-// record of 62 floats per vertex - position(3) normal(3) sh(48, planar: dc r,g,b then 15 r, 15 g,
-// 15 b) opacity-logit(1) log-scale(3) quaternion(4, r x y z).  Returns CPU tensors
+// The parsing lives in ply_reader.h (no torch in it).  Returns CPU tensors
 // (n, position[n,3], shs[n,48] interleaved per coefficient, opacity[n] after sigmoid,
 // cov3d[n,6] = upper triangle of R S^2 R^T).
-
-constexpr int kPlyFloats = 62;
-
-// Sigma from exp'd scales and a normalised quaternion, in the operation order of
-// computeCov3D (pybind.cpp:22-56): M = S * R in GLM's column-major product, Sigma = M^T * M.
-void cov3d_from(const float s[3], const float q[4], float out[6])
-{
-    const float r = q[0], x = q[1], y = q[2], z = q[3];
-    // R[c][k]: GLM column c, element k (the nine constructor arguments fill columns)
-    const float R[3][3] = {
-        { 1.f - 2.f * (y * y + z * z), 2.f * (x * y - r * z), 2.f * (x * z + r * y) },
-        { 2.f * (x * y + r * z), 1.f - 2.f * (x * x + z * z), 2.f * (y * z - r * x) },
-        { 2.f * (x * z - r * y), 2.f * (y * z + r * x), 1.f - 2.f * (x * x + y * y) } };
-    float M[3][3];   // M[c][k] = sum_j S[j][k] * R[c][j], S diagonal; the zero products are kept
-    for (int c = 0; c < 3; c++)
-        for (int k = 0; k < 3; k++) {
-            float acc[3];
-            for (int j = 0; j < 3; j++) acc[j] = (j == k ? s[k] : 0.0f) * R[c][j];
-            M[c][k] = acc[0] + acc[1] + acc[2];
-        }
-    auto sigma = [&](int c, int k) {   // (M^T * M)[c][k] = sum_j M[j][c]... in GLM order: Mt[j][k] * M[c][j]
-        return M[k][0] * M[c][0] + M[k][1] * M[c][1] + M[k][2] * M[c][2];
-    };
-    out[0] = sigma(0, 0); out[1] = sigma(0, 1); out[2] = sigma(0, 2);
-    out[3] = sigma(1, 1); out[4] = sigma(1, 2); out[5] = sigma(2, 2);
-}
-
 std::tuple<int, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> loadPly(const std::string& name)
 {
     std::ifstream file(name, std::ios::binary);
     if (!file.is_open()) throw std::runtime_error(std::string("Failed to open file: ") + name);
-    int n = 0;
-    bool header_done = false;
-    std::string tok;
-    while (file >> tok) {
-        if (tok == "vertex") {
-            file >> n;
-            if (n <= 0) throw std::runtime_error("Vertex number is not positive");
-        } else if (tok == "end_header") {
-            header_done = true;
-            file.get();   // the newline that ends the header
-            break;
-        }
-    }
-    if (!header_done) throw std::runtime_error("Cannot find end of header");
+    file.seekg(0, std::ios::end);
+    const std::streamoff size = file.tellg();
+    file.seekg(0, std::ios::beg);
+    if (size < 0) throw std::runtime_error(std::string("Failed to open file: ") + name);
+    // the count is bounded by the file's size before anything is allocated for it
+    const int n = fgs_ply::read_header(file, (uint64_t)size);
 
     auto opt = torch::TensorOptions().dtype(torch::kFloat32).device(torch::kCPU);
     torch::Tensor position = torch::empty({n, 3}, opt), shs = torch::empty({n, 48}, opt);
     torch::Tensor opacity = torch::empty({n}, opt), cov3d = torch::empty({n, 6}, opt);
-    float* pp = position.data_ptr<float>();
-    float* ps = shs.data_ptr<float>();
-    float* po = opacity.data_ptr<float>();
-    float* pc = cov3d.data_ptr<float>();
-
-    std::vector<float> rec(kPlyFloats);
-    for (int i = 0; i < n; i++) {
-        file.read(reinterpret_cast<char*>(rec.data()), kPlyFloats * sizeof(float));
-        if (!file) throw std::runtime_error("Unexpected end of file in vertex data");
-        const float* sh = rec.data() + 6;
-        std::memcpy(pp + 3 * (size_t)i, rec.data(), 3 * sizeof(float));
-        float* o = ps + 48 * (size_t)i;
-        o[0] = sh[0]; o[1] = sh[1]; o[2] = sh[2];
-        for (int j = 1; j < 16; j++) {           // planar rest coefficients -> interleaved RGB
-            o[3 * j + 0] = sh[3 + (j - 1)];
-            o[3 * j + 1] = sh[3 + 15 + (j - 1)];
-            o[3 * j + 2] = sh[3 + 30 + (j - 1)];
-        }
-        po[i] = 1.0f / (1.0f + std::exp(-rec[54]));
-        const float s[3] = { std::exp(rec[55]), std::exp(rec[56]), std::exp(rec[57]) };
-        // glm::normalize: v * (1 / sqrt(dot)), dot = (x*x + y*y) + (z*z + w*w)
-        const float* q0 = rec.data() + 58;
-        const float inv = 1.0f / std::sqrt((q0[0] * q0[0] + q0[1] * q0[1]) + (q0[2] * q0[2] + q0[3] * q0[3]));
-        const float q[4] = { q0[0] * inv, q0[1] * inv, q0[2] * inv, q0[3] * inv };
-        cov3d_from(s, q, pc + 6 * (size_t)i);
-    }
+    fgs_ply::read_records(file, n, position.data_ptr<float>(), shs.data_ptr<float>(), opacity.data_ptr<float>(),
+                          cov3d.data_ptr<float>());
     return std::make_tuple(n, position, shs, opacity, cov3d);
+}
+
+// No counterpart in the reference: clears the scan status that preprocess keeps for the current
+// stream of `like`'s device (fgs_reset_scan), the way back after a preprocess reported a negative
+// pair count.
+void reset_scan(torch::Tensor& like)
+{
+    need(like.is_cuda(), "reset_scan takes a GPU tensor that names the device");
+    DeviceScope scope(like);
+    fgs_check(fgs_reset_scan(current_stream(like)), "reset_scan");
 }
 
 } // namespace
@@ -281,4 +229,5 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     ops.def("render_16x16", &render<16, 16>, "tile ranges and alpha blending, 16x16 tiles");
     ops.def("render_32x16", &render<32, 16>, "tile ranges and alpha blending, 32x16 tiles");
     ops.def("render_32x32", &render<32, 32>, "tile ranges and alpha blending, 32x32 tiles");
+    ops.def("reset_scan", &reset_scan, "clear preprocess's scan status on the tensor's device and current stream");
 }

@@ -785,8 +785,19 @@ __global__ __launch_bounds__(kSharedWaves * kWave) __attribute__((amdgpu_waves_p
 #undef FGS_BLEND_PARAMS
 #undef FGS_BLEND_ARGS
 
-// How the colour sums are formed, for every blend launched after the setting (see fgs_set_colour_sums).
-std::atomic<int> g_colour_sums{FGS_COLOUR_SUMS_MATRIX_F16};
+// How the colour sums are formed by the entry points that do not say (see fgs_set_colour_sums).
+std::atomic<int> g_colour_sums{FGS_COLOUR_SUMS_FP32};
+
+// The mode of one call: what its flags ask for, else the process default.
+int colour_mode(int flags, int* mode, const char* who)
+{
+    if (flags & ~(FGS_BLEND_FP32 | FGS_BLEND_MATRIX_F16)) return fail(FGS_E_INVALID, "%s: unknown flags 0x%x", who, flags);
+    if ((flags & FGS_BLEND_FP32) && (flags & FGS_BLEND_MATRIX_F16))
+        return fail(FGS_E_INVALID, "%s: FGS_BLEND_FP32 and FGS_BLEND_MATRIX_F16 exclude each other", who);
+    *mode = (flags & FGS_BLEND_FP32) ? FGS_COLOUR_SUMS_FP32
+          : (flags & FGS_BLEND_MATRIX_F16) ? FGS_COLOUR_SUMS_MATRIX_F16 : g_colour_sums.load();
+    return FGS_OK;
+}
 
 int check_tile(int block_x, int block_y, int* sx, int* sy, const char* who)
 {
@@ -848,10 +859,12 @@ int ranges_impl(int block_x, int block_y, int num_rendered, int width, int heigh
 int blend_impl(int block_x, int block_y, int width, int height,
                const float* points_xy, const float* rgb_depth, const float* conic_opacity,
                const uint32_t* values_sorted, const int* ranges, const float bg[3],
-               uint8_t* out_u8, float* out_f32, void* stream, const char* who)
+               uint8_t* out_u8, float* out_f32, int flags, void* stream, const char* who)
 {
-    int sx = 0, sy = 0;
+    int sx = 0, sy = 0, mode = 0;
     int rc = check_tile(block_x, block_y, &sx, &sy, who);
+    if (rc != FGS_OK) return rc;
+    rc = colour_mode(flags, &mode, who);
     if (rc != FGS_OK) return rc;
     if (width <= 0 || height <= 0) return fail(FGS_E_INVALID, "%s: width/height must be positive", who);
     if (!ranges || !bg || (!out_u8 && !out_f32)) return fail(FGS_E_INVALID, "%s: null ranges, bg_color or output", who);
@@ -869,7 +882,7 @@ int blend_impl(int block_x, int block_y, int width, int height,
     rc = blend_shape(block_x, block_y, tiles_x, tiles_y, &shape);
     if (rc != FGS_OK) return rc;
     const bool few_waves = shape.few_waves;
-    const bool fp32 = g_colour_sums.load() == FGS_COLOUR_SUMS_FP32;
+    const bool fp32 = mode == FGS_COLOUR_SUMS_FP32;
 #define FGS_LAUNCH_BLEND(SX, SY)                                                                        \
     do {                                                                                                \
         auto kernel = fp32 ? (few_waves ? blend_kernel_few_waves<SX, SY, true> : blend_kernel<SX, SY, true>) \
@@ -899,17 +912,19 @@ int blend_impl(int block_x, int block_y, int width, int height,
 int render_impl(int block_x, int block_y, int num_rendered, int width, int height,
                 const float* points_xy, const float* rgb_depth, const float* conic_opacity,
                 const uint64_t* keys_sorted, const uint32_t* values_sorted,
-                int* ranges, const float bg[3], uint8_t* out_u8, float* out_f32, void* stream, const char* who)
+                int* ranges, const float bg[3], uint8_t* out_u8, float* out_f32, int flags, void* stream, const char* who)
 {
-    int sx = 0, sy = 0;
+    int sx = 0, sy = 0, mode = 0;
     int rc = check_tile(block_x, block_y, &sx, &sy, who);
+    if (rc != FGS_OK) return rc;
+    rc = colour_mode(flags, &mode, who);        // before anything is launched
     if (rc != FGS_OK) return rc;
     if (num_rendered > 0 && (!points_xy || !rgb_depth || !conic_opacity || !keys_sorted || !values_sorted))
         return fail(FGS_E_INVALID, "%s: null buffer", who);
     rc = ranges_impl(block_x, block_y, num_rendered, width, height, keys_sorted, ranges, stream, who);
     if (rc != FGS_OK) return rc;
     return blend_impl(block_x, block_y, width, height, points_xy, rgb_depth, conic_opacity, values_sorted, ranges,
-                      bg, out_u8, out_f32, stream, who);
+                      bg, out_u8, out_f32, flags, stream, who);
 }
 
 } // namespace
@@ -924,7 +939,7 @@ int render_impl(int block_x, int block_y, int num_rendered, int width, int heigh
         if (!out_color) return fgs::fail(FGS_E_INVALID, #NAME ": null out_color");                           \
         return fgs::render_impl(BX, BY, num_rendered, width, height, points_xy, rgb_depth, conic_opacity,    \
                                 gaussian_keys_sorted, gaussian_values_sorted, ranges, bg_color, out_color,   \
-                                nullptr, stream, #NAME);                                                     \
+                                nullptr, 0, stream, #NAME);                                                  \
     }
 
 FGS_DEFINE_RENDER(fgs_render_16x16, 16, 16)
@@ -939,7 +954,18 @@ extern "C" int fgs_render_f32(int block_x, int block_y, int num_rendered, int wi
 {
     return fgs::render_impl(block_x, block_y, num_rendered, width, height, points_xy, rgb_depth,
                             conic_opacity, gaussian_keys_sorted, gaussian_values_sorted, ranges, bg_color,
-                            out_color_u8, out_color_f32, stream, "fgs_render_f32");
+                            out_color_u8, out_color_f32, 0, stream, "fgs_render_f32");
+}
+
+extern "C" int fgs_render_ex(int block_x, int block_y, int num_rendered, int width, int height,
+                             const float* points_xy, const float* rgb_depth, const float* conic_opacity,
+                             const uint64_t* gaussian_keys_sorted, const uint32_t* gaussian_values_sorted,
+                             int* ranges, const float bg_color[3], uint8_t* out_color_u8, float* out_color_f32,
+                             int flags, void* stream)
+{
+    return fgs::render_impl(block_x, block_y, num_rendered, width, height, points_xy, rgb_depth,
+                            conic_opacity, gaussian_keys_sorted, gaussian_values_sorted, ranges, bg_color,
+                            out_color_u8, out_color_f32, flags, stream, "fgs_render_ex");
 }
 
 extern "C" int fgs_set_colour_sums(int mode)
@@ -951,14 +977,15 @@ extern "C" int fgs_set_colour_sums(int mode)
     return fgs::g_colour_sums.exchange(mode);
 }
 
-extern "C" const char* fgs_blend_kernel_name(int block_x, int block_y, int width, int height)
+extern "C" const char* fgs_blend_kernel_name(int block_x, int block_y, int width, int height, int flags)
 {
     using namespace fgs;
-    int sx = 0, sy = 0;
+    int sx = 0, sy = 0, mode = 0;
     if (check_tile(block_x, block_y, &sx, &sy, "fgs_blend_kernel_name") != FGS_OK || width <= 0 || height <= 0) return "";
+    if (colour_mode(flags, &mode, "fgs_blend_kernel_name") != FGS_OK) return "";
     BlendShape shape;
     if (blend_shape(block_x, block_y, (width + block_x - 1) / block_x, (height + block_y - 1) / block_y, &shape) != FGS_OK) return "";
-    const bool fp32 = g_colour_sums.load() == FGS_COLOUR_SUMS_FP32;
+    const bool fp32 = mode == FGS_COLOUR_SUMS_FP32;
 #define FGS_NAME(few, plain) (shape.few_waves ? (fp32 ? few ", true>" : few ", false>") : (fp32 ? plain ", true>" : plain ", false>"))
     if (shape.shared) return fp32 ? "tile_order_kernel + blend_kernel_shared<true>" : "tile_order_kernel + blend_kernel_shared<false>";
     if (sx == 1 && sy == 1) return FGS_NAME("blend_kernel_few_waves<1, 1", "blend_kernel<1, 1");
@@ -980,6 +1007,15 @@ extern "C" int fgs_blend(int block_x, int block_y, int width, int height,
                          uint8_t* out_color_u8, float* out_color_f32, void* stream)
 {
     return fgs::blend_impl(block_x, block_y, width, height, points_xy, rgb_depth, conic_opacity,
-                           gaussian_values_sorted, ranges, bg_color, out_color_u8, out_color_f32, stream, "fgs_blend");
+                           gaussian_values_sorted, ranges, bg_color, out_color_u8, out_color_f32, 0, stream, "fgs_blend");
+}
+
+extern "C" int fgs_blend_ex(int block_x, int block_y, int width, int height,
+                            const float* points_xy, const float* rgb_depth, const float* conic_opacity,
+                            const uint32_t* gaussian_values_sorted, const int* ranges, const float bg_color[3],
+                            uint8_t* out_color_u8, float* out_color_f32, int flags, void* stream)
+{
+    return fgs::blend_impl(block_x, block_y, width, height, points_xy, rgb_depth, conic_opacity,
+                           gaussian_values_sorted, ranges, bg_color, out_color_u8, out_color_f32, flags, stream, "fgs_blend_ex");
 }
 

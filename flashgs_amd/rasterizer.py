@@ -3,8 +3,9 @@
 through ``flash_gaussian_splatting.ops``, ``savePpm`` and ``render_scene``.
 
 Differences from the reference driver: the output image is allocated once instead of per frame,
-the too-many-pairs condition raises a real exception (``example.py:82`` raises a string), and the
-tile size is a constructor argument.
+the too-many-pairs condition raises a real exception (``example.py:82`` raises a string), a
+preprocess whose bounded waits gave up is launched once more after ``ops.reset_scan`` and raises
+``ScanGaveUp`` if that fails too, and the tile size is a constructor argument.
 """
 import json
 import os
@@ -78,7 +79,12 @@ class Camera:
 
 
 class TooManyPairs(RuntimeError):
-    pass
+    """More (tile, Gaussian) pairs than the key buffers hold (example.py:81-82)."""
+
+
+class ScanGaveUp(RuntimeError):
+    """A wait inside the preprocess launch ran into its poll limit, twice in a row: the pair
+    count came back negative although the frame was launched again on cleared scan status."""
 
 
 class Rasterizer:
@@ -120,18 +126,26 @@ class Rasterizer:
         tiles = ((camera.width + bx - 1) // bx) * ((camera.height + by - 1) // by)
         if tiles > self.MAX_NUM_TILES:
             raise ValueError("image needs %d tiles, MAX_NUM_TILES is %d" % (tiles, self.MAX_NUM_TILES))
-        self.curr_offset.zero_()
-        o.preprocess(scene.position, scene.shs, scene.opacity, scene.cov3d,
-                     camera.width, camera.height, bx, by,
-                     camera.position, camera.rotation,
-                     camera.focal_x, camera.focal_y, camera.zFar, camera.zNear,
-                     self.points_xy, self.rgb_depth, self.conic_opacity,
-                     self.gaussian_keys_unsorted, self.gaussian_values_unsorted, self.curr_offset)
-        # the one blocking device-to-host read of the frame (example.py:79)
-        self._offset_host.copy_(self.curr_offset, non_blocking=False)
-        num_rendered = int(self._offset_host[0])
+        for attempt in range(2):
+            self.curr_offset.zero_()
+            o.preprocess(scene.position, scene.shs, scene.opacity, scene.cov3d,
+                         camera.width, camera.height, bx, by,
+                         camera.position, camera.rotation,
+                         camera.focal_x, camera.focal_y, camera.zFar, camera.zNear,
+                         self.points_xy, self.rgb_depth, self.conic_opacity,
+                         self.gaussian_keys_unsorted, self.gaussian_values_unsorted, self.curr_offset)
+            # the one blocking device-to-host read of the frame (example.py:79)
+            self._offset_host.copy_(self.curr_offset, non_blocking=False)
+            num_rendered = int(self._offset_host[0])
+            if num_rendered >= 0:
+                break
+            # a bounded wait of the launch gave up: clear the scan status and launch once more
+            o.reset_scan(self.curr_offset)
         self.num_rendered = num_rendered
-        if num_rendered < 0 or num_rendered >= self.MAX_NUM_RENDERED:
+        if num_rendered < 0:
+            raise ScanGaveUp("preprocess gave up waiting for its scan over workgroups twice in a row "
+                             "(fgs_set_scan_spin_limit polls); the frame was not rendered")
+        if num_rendered >= self.MAX_NUM_RENDERED:
             raise TooManyPairs("Too many k-v pairs! (%d, capacity %d)" % (num_rendered, self.MAX_NUM_RENDERED))
         o.sort_gaussian(num_rendered, camera.width, camera.height, bx, by, self.list_sorting_space,
                         self.gaussian_keys_unsorted, self.gaussian_values_unsorted,

@@ -205,6 +205,15 @@ def config3(n=8_000_000):
     return _city_scene("cfg3_8M_8K", 3, n, 200.0, 7680, 4320, 70.0, big_fraction=0.02)
 
 
+def config3_dense(n=8_000_000, base=None):
+    """The 8K scene with every splat five times as large (covariances x 25): more than 100M pairs and
+    hundreds of tiles with more than 8192 of them, the regime the 8K configuration is meant to
+    stress.  `base` may be an already generated config3 scene of the same n, whose arrays are shared."""
+    sc = base if base is not None else config3(n)
+    return Scene("cfg3_dense_8M_8K", sc.position, sc.shs, sc.opacity, (sc.cov3d * np.float32(25.0)).astype(np.float32),
+                 list(sc.cameras))
+
+
 def config4(n=2_000_000, width=1920, height=1080, n_poses=60):
     """Orbit of 60 poses (radius 30, height 5, 6 degree steps) around the cluster scene; 10 % of
     the Gaussians are 100:1 anisotropic and lie within 1 unit of the camera path."""
@@ -230,7 +239,7 @@ def config4(n=2_000_000, width=1920, height=1080, n_poses=60):
     return _finish("cfg4_2M_orbit_%dx%d" % (width, height), rng, means, log_scales, 0.0, 2.0, cams)
 
 
-CONFIGS = {0: config0, 1: config1, 2: config2, 3: config3, 4: config4}
+CONFIGS = {0: config0, 1: config1, 2: config2, 3: config3, 4: config4, 5: config3_dense}
 
 
 def make(config, **kw):

@@ -48,14 +48,22 @@ extern "C" {
  * unchecked like the reference (preprocess.cu:330,395).
  *
  * The call is asynchronous on `stream`.  The library keeps a small scratch for the scan over
- * workgroups per (device, stream), allocated on the first call on that stream and grown when a
- * larger P arrives - the only times the call synchronises - so calls on different streams of one
- * device may overlap in time.  Nothing on the host changes from launch to launch, so a launch can
- * be captured in a HIP graph and replayed; a stream that is being captured and has no (large
- * enough) scratch yet cannot allocate one and uses the built-in scan status of
- * fgs_preprocess_static, with its limits.  Every wait inside the launch is bounded
- * (fgs_set_scan_spin_limit); if one ever gives up, *curr_offset ends negative and the keys are
- * not to be used.
+ * workgroups per (device, stream), allocated on the first call on that stream, so calls on
+ * different streams of one device may overlap in time.  When a larger P arrives a larger scratch
+ * is allocated and the earlier one is kept, never freed (32 bytes per 256 Gaussians it was sized
+ * for), because a HIP graph captured on the stream holds its address.  Nothing on the host changes
+ * from launch to launch, so a launch can be captured in a HIP graph and replayed, also after
+ * larger eager calls on the same stream; a stream that is being captured and has no (large enough)
+ * scratch yet cannot allocate one and uses the built-in scan status of fgs_preprocess_static, with
+ * its limits.
+ *
+ * Every wait inside the launch is bounded (fgs_set_scan_spin_limit).  If one ever gives up,
+ * *curr_offset ends negative (INT_MIN) and keys, values and attribute rows are not to be used.
+ * When it was the scan itself that gave up, the scratch is left marked unusable: every later
+ * fgs_preprocess on that stream (and every fgs_preprocess_static on that device, if it was the
+ * built-in scratch) reports a negative count too, at once and without touching anything, until
+ * fgs_reset_scan has been called on the stream.  So the caller's recovery is: see a negative
+ * count, call fgs_reset_scan(stream), zero *curr_offset, call fgs_preprocess again.
  */
 int fgs_preprocess(int P,
                    const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
@@ -109,9 +117,8 @@ size_t fgs_get_sort_buffer_size(int num_rendered);
  * csrc/cuda_rasterizer/render.cu:549-608): zero `ranges`, find each tile's [start,end) in the
  * sorted keys, blend front to back and write out_color u8[H,W,3].  `ranges` int32[tiles,2] is
  * scratch that holds the tile ranges afterwards.  bg_color is a host array of 3 floats.
- * Exponent, alpha and transmittance are fp32; the colour sums take the weights alpha*T and the
- * colours rounded to f16 (products and sums in fp32), so a pixel's colour is within 2^-10 of
- * itself of the all-fp32 sum; colours beyond +-65504 are drawn as +-65504.
+ * All arithmetic is fp32, as in render.cu:40-52, unless the process default was changed with
+ * fgs_set_colour_sums (fgs_render_ex / fgs_blend_ex choose per call).
  * A frame of at most 8192 16x16 tiles first ranks its tiles by list length into a table the
  * library keeps per (device, stream) (32 KB, allocated on the first such call on that stream),
  * and the rest of a list of more than 768 entries is blended in four runs that each stop on
@@ -159,27 +166,47 @@ int fgs_blend(int block_x, int block_y, int width, int height,
               uint8_t* out_color_u8, float* out_color_f32, void* stream);
 
 /*
- * No counterpart in the reference.  Name of the kernel(s) fgs_blend / fgs_render_* launch on the
- * current device for this tile and frame size (the choice depends on how many tiles the frame has
- * against what the chip holds at once), as a profiler lists them; "" for an unsupported tile size.
- * Lets a benchmark attribute its figures to the kernel that ran.
- */
-const char* fgs_blend_kernel_name(int block_x, int block_y, int width, int height);
-
-/*
- * No counterpart in the reference.  How the blend forms its colour sums C += (alpha T) c, for
- * every blend launched after the call (process-wide); returns the previous mode, -1 for an
- * unknown one.
- *   FGS_COLOUR_SUMS_MATRIX_F16 (default): on the matrix unit; the weights alpha T and the colours
- *     are rounded to f16, products and sums are fp32: a pixel's colour is within 2^-10 of itself
- *     of the all-fp32 sum, colours beyond +-65504 are drawn as +-65504.
- *   FGS_COLOUR_SUMS_FP32: by fp32 multiply-add, operation for operation what render.cu:40-52
- *     does; about a tenth slower on a 4K frame.
+ * No counterpart in the reference.  How a blend forms its colour sums C += (alpha T) c.
+ *   FGS_COLOUR_SUMS_FP32 (default): by fp32 multiply-add, operation for operation what
+ *     render.cu:40-52 does.
+ *   FGS_COLOUR_SUMS_MATRIX_F16 (opt-in, about a fifth faster in the blend of a 4K frame): on the
+ *     matrix unit; the weights alpha T and the colours are rounded to f16, products and sums are
+ *     fp32: a pixel's colour is within 2^-10 of itself of the all-fp32 sum.  Colours beyond
+ *     +-65504 are drawn as +-65504 and opacities above 3.97 as 3.97; a conic that is not positive
+ *     definite (its exponent grows without bound away from the centre) can push a weight past
+ *     f16's range, which the fp32 mode does not have - keep such inputs on the default.
  * Exponent, alpha and transmittance are fp32 in both.
+ *
+ * fgs_set_colour_sums sets the process-wide default, which the entry points without a flags
+ * argument use at the time of the call (fgs_render_<bx>x<by>, fgs_render_f32, fgs_blend); it
+ * returns the previous default, -1 for an unknown mode.  A caller that shares the process with
+ * other renderers passes the mode per call instead: fgs_render_ex and fgs_blend_ex are
+ * fgs_render_f32 and fgs_blend with a flags argument, 0 = the process default, FGS_BLEND_FP32 or
+ * FGS_BLEND_MATRIX_F16 = that mode whatever the default is.
  */
 #define FGS_COLOUR_SUMS_MATRIX_F16 0
 #define FGS_COLOUR_SUMS_FP32       1
 int fgs_set_colour_sums(int mode);
+
+#define FGS_BLEND_FP32        1
+#define FGS_BLEND_MATRIX_F16  2
+int fgs_render_ex(int block_x, int block_y, int num_rendered, int width, int height,
+                  const float* points_xy, const float* rgb_depth, const float* conic_opacity,
+                  const uint64_t* gaussian_keys_sorted, const uint32_t* gaussian_values_sorted,
+                  int* ranges, const float bg_color[3], uint8_t* out_color_u8, float* out_color_f32,
+                  int flags, void* stream);
+int fgs_blend_ex(int block_x, int block_y, int width, int height,
+                 const float* points_xy, const float* rgb_depth, const float* conic_opacity,
+                 const uint32_t* gaussian_values_sorted, const int* ranges, const float bg_color[3],
+                 uint8_t* out_color_u8, float* out_color_f32, int flags, void* stream);
+
+/*
+ * No counterpart in the reference.  Name of the kernel(s) a blend with these flags launches on
+ * the current device for this tile and frame size (the choice depends on how many tiles the frame
+ * has against what the chip holds at once), as a profiler lists them; "" for an unsupported tile
+ * size or unknown flags.  Lets a benchmark attribute its figures to the kernel that ran.
+ */
+const char* fgs_blend_kernel_name(int block_x, int block_y, int width, int height, int flags);
 
 /*
  * Host-side camera set-up used by fgs_preprocess (preprocess.cu:420-448,461-466), exposed so
@@ -199,10 +226,24 @@ void fgs_camera_matrices(const float cam_position[3], const float cam_rotation[9
  */
 unsigned fgs_set_scan_spin_limit(unsigned polls);
 
+/*
+ * No counterpart in the reference.  Clears the scan status that fgs_preprocess keeps for `stream`
+ * on the current device, and the built-in one of fgs_preprocess_static on that device, with a
+ * small kernel enqueued on `stream` (so it is ordered after the launches already on it and may be
+ * captured).  Needed only after a preprocess that reported a negative pair count, see there;
+ * harmless otherwise.  Must not overlap a preprocess launch that uses the same scan status from
+ * another stream.
+ */
+int fgs_reset_scan(void* stream);
+
 /* Message of the last failing call on this thread ("" if none). */
 const char* fgs_last_error(void);
 
-/* ABI version of this header: bumped when a signature changes. */
+/*
+ * ABI version of this header as major * 1000 + minor: the major number changes when an existing
+ * signature or default changes, the minor one when entry points are added.
+ */
+#define FGS_ABI_VERSION 2000
 int fgs_abi_version(void);
 
 #ifdef __cplusplus

@@ -171,8 +171,9 @@ inline void get_rect(float px, float py, int width, int height, int gx, int gy, 
 {
     rmin[0] = imin(gx, imax(0, f2i_sat((px - (float)width) / (float)bx)));
     rmin[1] = imin(gy, imax(0, f2i_sat((py - (float)height) / (float)by)));
-    rmax[0] = imin(gx, imax(0, f2i_sat((px + (float)width) / (float)bx) + 1));
-    rmax[1] = imin(gy, imax(0, f2i_sat((py + (float)height) / (float)by) + 1));
+    /* the "+ 1" wraps at INT_MAX as the device's integer add does (the rectangle is then empty) */
+    rmax[0] = imin(gx, imax(0, (int)((uint32_t)f2i_sat((px + (float)width) / (float)bx) + 1u)));
+    rmax[1] = imin(gy, imax(0, (int)((uint32_t)f2i_sat((py + (float)height) / (float)by) + 1u)));
 }
 
 /* ---- preprocess.cu:103-143 ----------------------------------------------- */
@@ -544,7 +545,7 @@ int fgs_oracle_preprocess(int P, const float* positions, const float* shs,
     for (int t = 0; t < T; t++) {
         int64_t dst = base + off[t];
         int64_t n = (int64_t)tkeys[t].size();
-        if (dst >= capacity) continue;
+        if (dst >= capacity || n == 0) continue;        // (an empty vector's data() may be null)
         if (dst + n > capacity) n = capacity - dst;
         memcpy(keys_unsorted + dst, tkeys[t].data(), (size_t)n * 8);
         memcpy(values_unsorted + dst, tvals[t].data(), (size_t)n * 4);

@@ -58,16 +58,18 @@ def sort(num, width, height, keys, values, block=(16, 16), space_for=None):
     return ks, vs
 
 
-def render(num, width, height, points_xy, rgb_depth, conic_opacity, ks, vs, bg, block=(16, 16), f32=True):
+def render(num, width, height, points_xy, rgb_depth, conic_opacity, ks, vs, bg, block=(16, 16), f32=True, flags=None):
+    """fgs_render_f32 (or the plain fgs_render_<bx>x<by> with f32=False); with `flags` (cabi.BLEND_*)
+    fgs_render_ex, which chooses the colour-sum mode for this call."""
     gx, gy = (width + block[0] - 1) // block[0], (height + block[1] - 1) // block[1]
     ranges = torch.full((gx * gy, 2), -7, device=DEV, dtype=torch.int32)
     out_u8 = torch.full((height, width, 3), 77, device=DEV, dtype=torch.uint8)
     out_f32 = torch.full((height, width, 3), -1.0, device=DEV, dtype=torch.float32) if f32 else None
     st = torch.cuda.current_stream().cuda_stream
-    if f32:
+    if f32 or flags is not None:
         cabi.render_f32(block[0], block[1], num, width, height, points_xy.data_ptr(), rgb_depth.data_ptr(),
                         conic_opacity.data_ptr(), ks.data_ptr(), vs.data_ptr(), ranges.data_ptr(), bg,
-                        out_u8.data_ptr(), out_f32.data_ptr(), st)
+                        out_u8.data_ptr(), out_f32.data_ptr() if f32 else 0, st, flags=flags)
     else:
         cabi.render(block[0], block[1], num, width, height, points_xy.data_ptr(), rgb_depth.data_ptr(),
                     conic_opacity.data_ptr(), ks.data_ptr(), vs.data_ptr(), ranges.data_ptr(), bg,

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), "libflashgs_hip.so does not export %s" % name
         assert name in cabi.SIGNATURES, "flashgs_amd/cabi.py has no binding for %s" % name
-    assert cabi.load().fgs_abi_version() == 1
+    assert cabi.load().fgs_abi_version() == 2000       # FGS_ABI_VERSION of the header: major * 1000 + minor
 
 
 def test_sort_buffer_size_is_monotonic_and_bounded():
@@ -81,10 +81,18 @@ def test_bad_arguments_are_rejected_before_any_launch():
 def test_colour_sums_switch_round_trips_and_rejects_unknown_modes():
     prev = cabi.set_colour_sums(cabi.COLOUR_SUMS_FP32)
     try:
-        assert prev in (cabi.COLOUR_SUMS_MATRIX_F16, cabi.COLOUR_SUMS_FP32)
+        assert prev == cabi.COLOUR_SUMS_FP32         # the library default is the reference's arithmetic
         assert cabi.set_colour_sums(cabi.COLOUR_SUMS_MATRIX_F16) == cabi.COLOUR_SUMS_FP32
         with pytest.raises(RuntimeError, match="unknown"):
             cabi.set_colour_sums(7)
         assert cabi.set_colour_sums(cabi.COLOUR_SUMS_MATRIX_F16) == cabi.COLOUR_SUMS_MATRIX_F16
     finally:
         cabi.set_colour_sums(prev)
+
+
+def test_per_call_blend_flags_are_checked_on_the_host():
+    # unknown bits and both modes at once are rejected before anything is launched
+    for flags in (4, 8, cabi.BLEND_FP32 | cabi.BLEND_MATRIX_F16):
+        _raises("(-1)", cabi.blend, 16, 16, 64, 64, 256, 256, 256, 256, 256, [0, 0, 0], 256, 0, 0, flags)
+        _raises("(-1)", cabi.render_f32, 16, 16, 0, 64, 64, 0, 0, 0, 0, 0, 256, [0, 0, 0], 256, 0, 0, flags)
+        assert cabi.blend_kernel_name(16, 16, 64, 64, flags) == ""

@@ -10,10 +10,12 @@ pytestmark = pytest.mark.gpu
 
 IMG_MAX_ABS = 2e-3
 IMG_PSNR_DB = 55.0
-# The colour sums of the blend take weights and colours rounded to f16 (products and sums in fp32):
-# a pixel's colour is within 2^-10 of itself of the oracle's, which moves the few 8-bit values that
-# lie that close to a step of the encode by one.
-IMG_U8_FRACTION = 0.02
+# 8-bit values that lie within the exponent's rounding of a step of the encode move by one.
+IMG_U8_FRACTION = 0.01
+# With the colour sums on the matrix unit (opt-in) weights and colours are rounded to f16 (products
+# and sums in fp32): a pixel's colour is within 2^-10 of itself of the oracle's, which moves a few
+# more of those 8-bit values.
+IMG_U8_FRACTION_F16 = 0.02
 
 
 def _oracle_frame(oracle, sc, cam, capacity, block=(16, 16), bg=(0, 0, 0), sentinel=0.0):
@@ -54,19 +56,30 @@ def _check_frame(oracle, sc, cam, capacity, block=(16, 16), bg=(0, 0, 0)):
     assert np.array_equal(gp.u64(ks)[:K], ref["ks"])
     assert np.array_equal(gp.u32(vs)[:K], ref["vs"])
 
+    # the library default: every operation of the blend in fp32, as render.cu:40-52
     rg, u8, f32 = gp.render(K, cam.width, cam.height, got["points_xy"], got["rgb_depth"], got["conic_opacity"],
                             ks, vs, bg, block)
     assert np.array_equal(rg.cpu().numpy(), ref["ranges"])
     f32 = f32.cpu().numpy()
     err = np.abs(f32 - ref["f32"])
     assert err.max() <= IMG_MAX_ABS, "max abs image error %g" % err.max()
-    # pixel by pixel: the f16 operands of the colour sums cost at most 2^-10 of the colour itself
-    over = err - (2.0 ** -10 * np.abs(ref["f32"]) + 2e-4)
-    assert over.max() <= 0, "a pixel is %g further from the oracle than f16 colour operands explain" % over.max()
     assert gp.psnr(f32, ref["f32"]) > IMG_PSNR_DB
     d8 = np.abs(u8.cpu().numpy().astype(np.int16) - ref["u8"].astype(np.int16))
     assert d8.max() <= 1, "8-bit image differs by more than one step"
     assert (d8 > 0).mean() < IMG_U8_FRACTION
+    # the opt-in mode with the colour sums on the matrix unit, chosen for this call only
+    from flashgs_amd import cabi
+    _, u8h, f16 = gp.render(K, cam.width, cam.height, got["points_xy"], got["rgb_depth"], got["conic_opacity"],
+                            ks, vs, bg, block, flags=cabi.BLEND_MATRIX_F16)
+    f16 = f16.cpu().numpy()
+    err16 = np.abs(f16 - ref["f32"])
+    assert err16.max() <= IMG_MAX_ABS, "f16 colour operands: max abs image error %g" % err16.max()
+    # pixel by pixel: the f16 operands of the colour sums cost at most 2^-10 of the colour itself
+    over = err16 - (2.0 ** -10 * np.abs(ref["f32"]) + 2e-4)
+    assert over.max() <= 0, "a pixel is %g further from the oracle than f16 colour operands explain" % over.max()
+    assert gp.psnr(f16, ref["f32"]) > IMG_PSNR_DB
+    d8 = np.abs(u8h.cpu().numpy().astype(np.int16) - ref["u8"].astype(np.int16))
+    assert d8.max() <= 1 and (d8 > 0).mean() < IMG_U8_FRACTION_F16
     return ref
 
 
@@ -261,33 +274,73 @@ def test_start_offset_and_capacity_guard(oracle):
     assert np.all(gp.u64(keys)[cap:] == 0) and np.all(values.cpu().numpy()[cap:] == -1)   # nothing past the capacity
 
 
-def test_scan_waits_that_give_up_report_a_negative_count(oracle):
+def test_scan_that_gives_up_reports_a_negative_count_until_reset():
     """With the spin limit at 0 every wait of the preprocess launch that is not satisfied at its
-    first poll gives up: the kernel still runs to its end (no wave is left waiting), the pair
-    count comes back negative - which the sort refuses - and the next launch with the normal
-    limit is correct again, both entry points."""
+    first poll gives up: the kernel still runs to its end (no wave is left waiting) and the pair
+    count comes back negative, which the sort refuses.  The frame has more workgroups than the chip
+    holds at once, so some are dispatched only after the scanner has given up.  The scan status is
+    then marked unusable: the next launch - another scene, normal limit - reports a negative count
+    as well and writes nothing; after fgs_reset_scan both scenes come out right again.  Both entry
+    points (the allocated scan status and the built-in one)."""
     import gpu_pipeline as gp
+    import torch
     from flashgs_amd import cabi
-    sc = scenes.config0(n=120_000)
-    cam = sc.cameras[0]
-    sd = gp.SceneOnDevice(sc)
-    good = gp.preprocess(sd, cam, 1 << 20)
-    K = good["num_rendered"]
-    assert K > 100_000
+    big = scenes.config0(n=1_200_000)            # 4689 workgroups
+    other = scenes.config1(n=300_000)
+    cam, cam_o = big.cameras[0], other.cameras[0]
+    sd, sd_o = gp.SceneOnDevice(big), gp.SceneOnDevice(other)
+    cap = 1 << 22
+    good, good_o = gp.preprocess(sd, cam, cap), gp.preprocess(sd_o, cam_o, cap)
+    K, K_o = good["num_rendered"], good_o["num_rendered"]
+    assert K > 1_000_000 and K_o > 100_000
+    st = torch.cuda.current_stream().cuda_stream
     for static in (False, True):
         previous = cabi.set_scan_spin_limit(0)
         try:
-            bad = gp.preprocess(sd, cam, 1 << 20, static=static)
+            bad = gp.preprocess(sd, cam, cap, static=static)
         finally:
             assert cabi.set_scan_spin_limit(previous) == 0
         assert previous == 1 << 22
         assert bad["num_rendered"] < 0
         with pytest.raises(RuntimeError, match="negative"):
             gp.sort(bad["num_rendered"], cam.width, cam.height, bad["keys"], bad["values"])
-        again = gp.preprocess(sd, cam, 1 << 20, static=static)
-        assert again["num_rendered"] == K
-        assert np.array_equal(gp.u64(again["keys"])[:K], gp.u64(good["keys"])[:K])
-        assert np.array_equal(gp.u32(again["values"])[:K], gp.u32(good["values"])[:K])
+        # sticky: another scene with the normal limit is refused at once and nothing is written
+        stuck = gp.preprocess(sd_o, cam_o, cap, sentinel=-3.5, static=static)
+        assert stuck["num_rendered"] < 0
+        assert not gp.u64(stuck["keys"]).any()
+        assert np.all(stuck["rgb_depth"].cpu().numpy() == -3.5)
+        cabi.reset_scan(st)
+        for scene_d, c, want, n in ((sd_o, cam_o, good_o, K_o), (sd, cam, good, K), (sd_o, cam_o, good_o, K_o)):
+            again = gp.preprocess(scene_d, c, cap, static=static)
+            assert again["num_rendered"] == n
+            assert np.array_equal(gp.u64(again["keys"])[:n], gp.u64(want["keys"])[:n])
+            assert np.array_equal(gp.u32(again["values"])[:n], gp.u32(want["values"])[:n])
+
+
+def test_rasterizer_relaunches_once_after_a_scan_that_gave_up():
+    """Rasterizer.forward clears the scan status and launches the frame once more when the pair
+    count comes back negative; with the waits still failing it raises ScanGaveUp, not TooManyPairs."""
+    import gpu_pipeline as gp
+    import torch
+    from flashgs_amd import cabi
+    from flashgs_amd.rasterizer import Camera, Rasterizer, ScanGaveUp, Scene
+    sc = scenes.config0(n=400_000)
+    scene = Scene(torch.device(gp.DEV)).from_arrays(sc.position, sc.shs, sc.opacity, sc.cov3d)
+    cam = Camera.from_synthetic(sc.cameras[0])
+    rast = Rasterizer(scene, 1 << 21, 1 << 14)
+    bg = torch.zeros(3)
+    want = rast.forward(scene, cam, bg).clone()
+    K = rast.num_rendered
+    # leave the stream's scan status marked unusable, as a scan that gave up does
+    previous = cabi.set_scan_spin_limit(0)
+    try:
+        with pytest.raises(ScanGaveUp):
+            rast.forward(scene, cam, bg)
+    finally:
+        cabi.set_scan_spin_limit(previous)
+    # the status is still marked; forward recovers by itself
+    got = rast.forward(scene, cam, bg)
+    assert rast.num_rendered == K and torch.equal(got, want)
 
 
 def test_preprocess_replayed_from_a_captured_graph():
@@ -333,6 +386,61 @@ def test_preprocess_replayed_from_a_captured_graph():
         for _ in range(replay + 1):
             gp.preprocess(small, cam, 1 << 16)
         torch.cuda.synchronize()
+
+
+def test_captured_preprocess_survives_a_larger_eager_call_on_its_stream():
+    """Warm-up, capture, then a larger P on the same stream: the stream gets a larger scan status,
+    and the one whose address the captured launch holds must stay alive and consistent.  Replays
+    before and after the larger call give the eager result."""
+    import gpu_pipeline as gp
+    import torch
+    from flashgs_amd import cabi
+    small = scenes.config0(n=70_000)
+    large = scenes.config0(n=1_200_000)          # 4689 workgroups: more than the first allocation holds
+    cam = small.cameras[0]
+    sd, sd_large = gp.SceneOnDevice(small), gp.SceneOnDevice(large)
+    cap = 1 << 22
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        eager = gp.preprocess(sd, cam, cap)                 # allocates the stream's scan status
+    K = eager["num_rendered"]
+    n = sd.n
+    xy = torch.zeros((n, 2), device=gp.DEV); rgb = torch.zeros((n, 4), device=gp.DEV); co = torch.zeros((n, 4), device=gp.DEV)
+    keys = torch.zeros(cap, device=gp.DEV, dtype=torch.int64)
+    values = torch.zeros(cap, device=gp.DEV, dtype=torch.int32)
+    off = torch.zeros(1, device=gp.DEV, dtype=torch.int32)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        off.zero_()
+        cabi.preprocess(n, sd.position.data_ptr(), sd.shs.data_ptr(), sd.opacity.data_ptr(), sd.cov3d.data_ptr(),
+                        cam.width, cam.height, 16, 16, cam.position, cam.rotation, cam.focal_x, cam.focal_y,
+                        cam.zFar, cam.zNear, xy.data_ptr(), rgb.data_ptr(), co.data_ptr(),
+                        keys.data_ptr(), values.data_ptr(), off.data_ptr(), cap, torch.cuda.current_stream().cuda_stream)
+
+    def replay_and_check(what):
+        keys.zero_(); values.zero_()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            graph.replay()
+        torch.cuda.synchronize()
+        assert int(off.cpu()[0]) == K, what
+        assert np.array_equal(gp.u64(keys)[:K], gp.u64(eager["keys"])[:K]), what
+        assert np.array_equal(gp.u32(values)[:K], gp.u32(eager["values"])[:K]), what
+
+    replay_and_check("replay before the larger call")
+    with torch.cuda.stream(side):
+        big1 = gp.preprocess(sd_large, cam, cap)            # the stream moves to a larger scan status
+    replay_and_check("replay after the larger call")
+    with torch.cuda.stream(side):
+        big2 = gp.preprocess(sd_large, cam, cap)
+    replay_and_check("second replay after the larger call")
+    Kl = big1["num_rendered"]
+    assert Kl > 1_000_000 and big2["num_rendered"] == Kl
+    assert np.array_equal(gp.u64(big1["keys"])[:Kl], gp.u64(big2["keys"])[:Kl])
+    ref_large = gp.preprocess(sd_large, cam, cap)           # on the default stream, its own scan status
+    assert np.array_equal(gp.u64(big1["keys"])[:Kl], gp.u64(ref_large["keys"])[:Kl])
 
 
 def test_sort_and_render_replayed_from_a_captured_graph():
@@ -514,17 +622,20 @@ def test_blend_long_lists_shared_between_waves(oracle):
     out = torch.full((H, W, 3), -1.0, device=gp.DEV, dtype=torch.float32)
     d = [gp.dev(a) for a in (xy_g, rgbd_g, co_g)]
     dv, dr = gp.dev(vals.view(np.int32)), gp.dev(ranges)
-    for _ in range(2):                                     # the second call reuses the tile ranking buffer
+    # the second call reuses the tile ranking buffer; then the same with the colour sums on the matrix unit
+    for flags, bound in ((None, 2e-4), (None, 2e-4), (cabi.BLEND_MATRIX_F16, 1e-3)):
         cabi.blend(16, 16, W, H, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), dv.data_ptr(), dr.data_ptr(),
-                   bg, 0, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+                   bg, 0, out.data_ptr(), torch.cuda.current_stream().cuda_stream, flags=flags)
         torch.cuda.synchronize()
         err = np.abs(out.cpu().numpy() - ref)
-        assert err.max() <= 1e-3, "max abs image error %g" % err.max()    # 1e-4 (runs) + 2^-10 of a colour
+        # 1e-4 for the runs that stop on their own T, plus 2^-10 of a colour with f16 operands
+        assert err.max() <= bound, "max abs image error %g (flags %r)" % (err.max(), flags)
 
 
-def _blend_lists(oracle, lists, W, H, bg, seed, colour_hi=1.5):
+def _blend_lists(oracle, lists, W, H, bg, seed, colour_hi=1.5, flags=None):
     """Builds the attribute tensors and ranges for hand-made per-tile lists (tile, length, opacity),
-    blends them with fgs_blend and with the oracle; returns (GPU float image, oracle float image)."""
+    blends them with fgs_blend (fgs_blend_ex when `flags` is given) and with the oracle; returns
+    (GPU float image, oracle float image)."""
     import gpu_pipeline as gp
     from flashgs_amd import cabi
     import torch
@@ -556,19 +667,20 @@ def _blend_lists(oracle, lists, W, H, bg, seed, colour_hi=1.5):
     d = [gp.dev(a) for a in (xy, rgbd, co)]
     dv, dr = gp.dev(vals.view(np.int32)), gp.dev(ranges)
     cabi.blend(16, 16, W, H, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), dv.data_ptr(), dr.data_ptr(),
-               bg, 0, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+               bg, 0, out.data_ptr(), torch.cuda.current_stream().cuda_stream, flags=flags)
     torch.cuda.synchronize()
     return out.cpu().numpy(), ref
 
 
 @pytest.mark.parametrize("W,H", [(320, 240), (3840, 400)])       # the kernel of small frames and the one of large frames
 def test_blend_faint_weights_keep_their_relative_accuracy(oracle, W, H):
-    """The colour sums take their weights as f16.  Lists of thousands of Gaussians whose weights
+    """With FGS_BLEND_MATRIX_F16 the colour sums take their weights as f16.  Lists of thousands of Gaussians whose weights
     alpha*T lie between 1e-8 and 1e-5, far below f16's smallest normal number 6e-5, still add up to
     colours that are right to 2^-10 of themselves: the weights are scaled before the conversion."""
     gx = (W + 15) // 16
     lists = [(t, 1500 + 37 * (t % 5), op) for t, op in zip(range(0, 12 * gx, gx + 3), [1e-5, 3e-6, 1e-6, 3e-7, 1e-7, 1e-8] * 2)]
-    got, ref = _blend_lists(oracle, lists, W, H, (0.0, 0.0, 0.0), seed=5)
+    from flashgs_amd import cabi
+    got, ref = _blend_lists(oracle, lists, W, H, (0.0, 0.0, 0.0), seed=5, flags=cabi.BLEND_MATRIX_F16)
     lit = ref > 0
     assert lit.any() and ref[lit].max() < 0.05                      # faint sums, nothing near 1
     assert np.all(np.abs(got - ref)[lit] <= 2.0 ** -10 * ref[lit] + 1e-9)
@@ -576,19 +688,22 @@ def test_blend_faint_weights_keep_their_relative_accuracy(oracle, W, H):
 
 
 def test_blend_colours_up_to_the_f16_range(oracle):
-    """Colours far above 1 (up to 6e4, just inside f16) blend like any other: within 2^-10 of the
-    pixel's own colour."""
+    """Colours far above 1 (up to 6e4, just inside f16) blend like any other with f16 operands:
+    within 2^-10 of the pixel's own colour."""
+    from flashgs_amd import cabi
     lists = [(t, 40 + t, 0.3) for t in range(0, 300, 7)]
-    got, ref = _blend_lists(oracle, lists, 320, 240, (0.1, 0.2, 0.3), seed=9, colour_hi=6.0e4)
+    got, ref = _blend_lists(oracle, lists, 320, 240, (0.1, 0.2, 0.3), seed=9, colour_hi=6.0e4, flags=cabi.BLEND_MATRIX_F16)
     assert ref.max() > 1.0e4
     assert np.all(np.abs(got - ref) <= 2.0 ** -10 * np.abs(ref) + 1e-4)
 
 
 @pytest.mark.parametrize("W,H,block", [(1280, 720, (16, 16)), (5120, 2880, (16, 16)), (1000, 600, (32, 16)), (1000, 600, (32, 32))])
-def test_fp32_colour_sums_mode(oracle, W, H, block):
-    """fgs_set_colour_sums(FGS_COLOUR_SUMS_FP32): the colour sums by fp32 multiply-add.  The image is
-    then as close to the oracle as the exponent's evaluation order allows, far inside the f16 bound
-    of the default mode, on the kernel of small frames, the one of large frames and both wide tiles."""
+def test_colour_sum_modes_per_call_and_by_default(oracle, W, H, block):
+    """The colour sums by fp32 multiply-add (the default) and on the matrix unit with f16 operands
+    (FGS_BLEND_MATRIX_F16), on the kernel of small frames, the one of large frames and both wide
+    tiles.  The fp32 image is as close to the oracle as the exponent's evaluation order allows, far
+    inside the f16 bound.  A per-call flag wins over the process default; the entry points without
+    flags follow fgs_set_colour_sums."""
     import gpu_pipeline as gp
     from flashgs_amd import cabi
     sc = scenes.config0(n=60_000)
@@ -603,22 +718,30 @@ def test_fp32_colour_sums_mode(oracle, W, H, block):
     got = gp.preprocess(gp.SceneOnDevice(sc), cam, 1 << 22, block=block)
     assert got["num_rendered"] == K
     ks, vs = gp.sort(K, W, H, got["keys"], got["values"], block)
-    images = {}
-    prev = cabi.set_colour_sums(cabi.COLOUR_SUMS_FP32)
-    try:
-        for mode in (cabi.COLOUR_SUMS_FP32, cabi.COLOUR_SUMS_MATRIX_F16):
-            cabi.set_colour_sums(mode)
-            assert ("true" if mode == cabi.COLOUR_SUMS_FP32 else "false") in cabi.blend_kernel_name(block[0], block[1], W, H)
-            _, u8, f32 = gp.render(K, W, H, got["points_xy"], got["rgb_depth"], got["conic_opacity"], ks, vs, bg, block)
-            images[mode] = (u8.cpu().numpy(), f32.cpu().numpy())
-    finally:
-        cabi.set_colour_sums(prev)
-    err32 = np.abs(images[cabi.COLOUR_SUMS_FP32][1] - ref["f32"])
-    err16 = np.abs(images[cabi.COLOUR_SUMS_MATRIX_F16][1] - ref["f32"])
+
+    def image(flags):
+        _, u8, f32 = gp.render(K, W, H, got["points_xy"], got["rgb_depth"], got["conic_opacity"], ks, vs, bg, block, flags=flags)
+        return u8.cpu().numpy(), f32.cpu().numpy()
+
+    assert "true>" in cabi.blend_kernel_name(block[0], block[1], W, H)                # the default is fp32
+    assert "true>" in cabi.blend_kernel_name(block[0], block[1], W, H, cabi.BLEND_FP32)
+    assert "false>" in cabi.blend_kernel_name(block[0], block[1], W, H, cabi.BLEND_MATRIX_F16)
+    by_default, fp32, f16 = image(None), image(cabi.BLEND_FP32), image(cabi.BLEND_MATRIX_F16)
+    assert np.array_equal(by_default[1], fp32[1]) and np.array_equal(by_default[0], fp32[0])
+    assert not np.array_equal(fp32[1], f16[1])
+    err32, err16 = np.abs(fp32[1] - ref["f32"]), np.abs(f16[1] - ref["f32"])
     assert err32.max() <= 2e-4, "fp32 colour sums: max abs image error %g" % err32.max()
     assert err16.max() <= IMG_MAX_ABS and err32.mean() < err16.mean()
-    d8 = np.abs(images[cabi.COLOUR_SUMS_FP32][0].astype(np.int16) - ref["u8"].astype(np.int16))
+    d8 = np.abs(fp32[0].astype(np.int16) - ref["u8"].astype(np.int16))
     assert d8.max() <= 1 and (d8 > 0).mean() < 0.005
+    prev = cabi.set_colour_sums(cabi.COLOUR_SUMS_MATRIX_F16)
+    try:
+        assert prev == cabi.COLOUR_SUMS_FP32
+        assert "false>" in cabi.blend_kernel_name(block[0], block[1], W, H)
+        assert np.array_equal(image(None)[1], f16[1])                 # flag-less calls follow the process default ...
+        assert np.array_equal(image(cabi.BLEND_FP32)[1], fp32[1])     # ... a flag does not
+    finally:
+        cabi.set_colour_sums(prev)
 
 
 def test_ranges_kernel_against_searchsorted():
@@ -688,10 +811,8 @@ def test_config3_more_than_100M_pairs(oracle, config3_scene):
     pair count: the count is still the full one and nothing is written past the capacity
     (the reference would write out of bounds there, preprocess.cu:330,395; example.py:79-82 only
     checks afterwards)."""
-    import copy
     import gpu_pipeline as gp
-    sc = copy.copy(config3_scene)
-    sc.cov3d = (config3_scene.cov3d * np.float32(25.0)).astype(np.float32)
+    sc = scenes.config3_dense(base=config3_scene)
     cam = sc.cameras[0]
     ref = _check_frame(oracle, sc, cam, 1 << 27)
     K = ref["K"]

@@ -16,7 +16,8 @@ def ops():
 
 
 def test_operator_names(ops):
-    for name in ("loadPly", "preprocess", "sort_gaussian", "get_sort_buffer_size", "render_16x16", "render_32x16", "render_32x32"):
+    for name in ("loadPly", "preprocess", "sort_gaussian", "get_sort_buffer_size", "render_16x16", "render_32x16", "render_32x32",
+                 "reset_scan"):
         assert callable(getattr(ops, name))
     assert ops.get_sort_buffer_size(2 ** 20) >= 12 * 2 ** 20
     with pytest.raises(RuntimeError):
@@ -88,5 +89,11 @@ def test_load_ply_errors(ops, tmp_path):
         ops.loadPly(str(neg))
     short = tmp_path / "short.ply"
     short.write_bytes(b"ply\nelement vertex 2\nend_header\n" + b"\0" * 100)
-    with pytest.raises(RuntimeError):
+    with pytest.raises(RuntimeError, match="exceeds the 0 records"):
         ops.loadPly(str(short))
+    # a header may claim any count: it is checked against the file's size before anything is allocated
+    # (2^31 - 1 vertices would be 532 GB of tensors)
+    huge = tmp_path / "huge.ply"
+    huge.write_bytes(b"ply\nelement vertex 2147483647\nend_header\n" + b"\0" * (62 * 4 * 3))
+    with pytest.raises(RuntimeError, match="exceeds the 3 records"):
+        ops.loadPly(str(huge))

@@ -38,6 +38,63 @@ def test_static_entry_point_matches_the_allocating_one():
     _same(got, want, want["num_rendered"])
 
 
+def test_static_entry_point_allocates_nothing_and_runs_under_capture():
+    """What the entry point is for.  The first call on a fresh stream leaves the device's free
+    memory as it was (the allocating entry point takes its scan status there); the call can be
+    captured into a graph on a stream that has never run a preprocess, which fails if anything
+    allocates or synchronises; replays, alternating with eager static calls of another size on
+    another scene, give the allocating entry point's result every time."""
+    import gpu_pipeline as gp
+    import torch
+    from flashgs_amd import cabi
+    a, b = scenes.config0(n=200_000), scenes.config1(n=90_000)
+    cam, cam_b = a.cameras[0], b.cameras[0]
+    sd, sd_b = gp.SceneOnDevice(a), gp.SceneOnDevice(b)
+    cap = 1 << 22
+    want, want_b = gp.preprocess(sd, cam, cap), gp.preprocess(sd_b, cam_b, cap)
+    K, K_b = want["num_rendered"], want_b["num_rendered"]
+    n = sd.n
+    xy = torch.zeros((n, 2), device=gp.DEV); rgb = torch.zeros((n, 4), device=gp.DEV); co = torch.zeros((n, 4), device=gp.DEV)
+    keys = torch.zeros(cap, device=gp.DEV, dtype=torch.int64)
+    values = torch.zeros(cap, device=gp.DEV, dtype=torch.int32)
+    off = torch.zeros(1, device=gp.DEV, dtype=torch.int32)
+
+    def launch(stream):
+        cabi.preprocess(n, sd.position.data_ptr(), sd.shs.data_ptr(), sd.opacity.data_ptr(), sd.cov3d.data_ptr(),
+                        cam.width, cam.height, 16, 16, cam.position, cam.rotation, cam.focal_x, cam.focal_y,
+                        cam.zFar, cam.zNear, xy.data_ptr(), rgb.data_ptr(), co.data_ptr(),
+                        keys.data_ptr(), values.data_ptr(), off.data_ptr(), cap, stream, static=True)
+
+    def check(what):
+        torch.cuda.synchronize()
+        assert int(off.cpu()[0]) == K, what
+        assert np.array_equal(gp.u64(keys)[:K], gp.u64(want["keys"])[:K]), what
+        assert np.array_equal(gp.u32(values)[:K], gp.u32(want["values"])[:K]), what
+
+    fresh = torch.cuda.Stream()
+    fresh.wait_stream(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    launch(fresh.cuda_stream)
+    check("first static call on a fresh stream")
+    assert torch.cuda.mem_get_info()[0] == free_before, "the static entry point took device memory"
+
+    side = torch.cuda.Stream()                   # has never run a preprocess: nothing to fall back on but the built-in status
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        off.zero_()
+        launch(torch.cuda.current_stream().cuda_stream)
+    assert torch.cuda.mem_get_info()[0] <= free_before      # the graph object itself may hold memory; the library none
+    for replay in range(3):
+        keys.zero_(); values.zero_()
+        graph.replay()
+        check("replay %d" % replay)
+        got_b = gp.preprocess(sd_b, cam_b, cap, static=True)            # another scene and size on the same status
+        assert got_b["num_rendered"] == K_b
+        assert np.array_equal(gp.u64(got_b["keys"])[:K_b], gp.u64(want_b["keys"])[:K_b])
+
+
 def test_static_entry_point_rejects_what_its_status_cannot_hold():
     from flashgs_amd import cabi
     with pytest.raises(RuntimeError, match="exceeds"):
