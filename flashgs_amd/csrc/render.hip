@@ -202,7 +202,7 @@ constexpr int kGroups = kBatch / 4;
 // products and sums are fp32: the colour of a pixel differs from the all-fp32 sum by at most
 // 2^-10 of itself.  The weights are scaled by 2^14 (added to the exponent when it is tabulated,
 // taken out again with the result), which keeps them in f16's normal range down to 4e-9.
-// T itself never leaves fp32.  The template parameter kFp32 of the walk selects the other form.
+// T itself never leaves fp32.  This form is opt-in (FGS_BLEND_MATRIX_F16); walk_list_fp32 is the default.
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float float2_t __attribute__((ext_vector_type(2)));
@@ -286,9 +286,9 @@ struct LaneRole {
     static constexpr int kFx = 16 * SX, kGy = 16 * SY;
     static constexpr int kRec = kFx + kGy + 4;  // floats per staged Gaussian: F table, G table; padded so that the
                                                 // staging lanes, one record apart, write to different LDS banks
-    static constexpr int kGroupRec = 28;        // floats per group of four: cy x 4, 4 channels x 4 f16, (r, g, b, -) x 4 as fp32
+    static constexpr int kGroupRec = 12;        // floats per group of four: cy x 4, 4 channels x 4 f16
     static constexpr int kStage = kBatch * kRec + kGroups * kGroupRec;      // floats of a wave's staging area
-    uint32_t off_f, off_g, off_cy, off_colour;  // byte offsets into the staging area (fp32 colours: off_cy + 48)
+    uint32_t off_f, off_g, off_cy, off_colour;  // byte offsets into the staging area
     int stage_slot;                             // Gaussian lane%32 of the batch
     bool stage_g;                               // lanes 0-31 tabulate F, 32-63 G
     float xy[SX * SY][2][2];                    // X*Y of the quad's pixels, offsets from the tile centre
@@ -332,7 +332,7 @@ __device__ __forceinline__ void clear_quad(Quad& q)
 // distance from the start of the tile's list, so that the pairs are the reference's pairs.
 // Returns true when the walk ended at the tile-wide stop.  s_rec is this wave's staging area of
 // LaneRole::kStage floats.
-template <int SX, int SY, bool kFp32>
+template <int SX, int SY>
 __device__ __forceinline__ bool walk_list(
     const LaneRole<SX, SY>& role, float* s_rec,
     const uint32_t* __restrict__ point_list, int begin, int n,
@@ -395,7 +395,7 @@ __device__ __forceinline__ bool walk_list(
             const float curv = unused ? 0.0f : (stage_g ? nco.z : nco.x);
             const float lin = unused ? 0.0f : nco.y * (stage_g ? ex : ey);
             // (log2 of the opacity is held below 2 so that no scaled weight leaves f16's range)
-            const float w_log2 = kFp32 ? nco.w : (nco.w > 1.99f ? 1.99f : nco.w) + kWeightScaleLog2;
+            const float w_log2 = (nco.w > 1.99f ? 1.99f : nco.w) + kWeightScaleLog2;
             const float con = stage_g ? 0.0f : (unused ? -1.0e30f : w_log2 - (nco.y * ex) * ey);
             const float c0 = con + e * (curv * e + lin);
             const float c1 = -(2.0f * curv * e + lin);
@@ -413,15 +413,10 @@ __device__ __forceinline__ bool walk_list(
                 auto in_range = [&](float c) {          // NaN stays NaN; a slot past the end of the list holds no colour
                     return unused ? 0.0f : (c > kColourMax ? kColourMax : (c < -kColourMax ? -kColourMax : c));
                 };
-                if (!kFp32) {
-                    colour[0] = (_Float16)in_range(nrgb.x);
-                    colour[4] = (_Float16)in_range(nrgb.y);
-                    colour[8] = (_Float16)in_range(nrgb.z);
-                    colour[12] = (_Float16)0.0f;
-                }
-                if (kFp32)
-                    *reinterpret_cast<float4*>(stage_group + 12 + 4 * (stage_slot & 3)) =
-                        unused ? make_float4(0.f, 0.f, 0.f, 0.f) : make_float4(nrgb.x, nrgb.y, nrgb.z, 0.f);
+                colour[0] = (_Float16)in_range(nrgb.x);
+                colour[4] = (_Float16)in_range(nrgb.y);
+                colour[8] = (_Float16)in_range(nrgb.z);
+                colour[12] = (_Float16)0.0f;
             }
         }
         __builtin_amdgcn_wave_barrier();
@@ -442,31 +437,22 @@ __device__ __forceinline__ bool walk_list(
         auto fetch_group = [&](int g) {
             StagedGroup r;
             r.cy = lds_read<float4>(rec_bytes + off_cy + g * kGroupRec * 4);
-            r.colour = kFp32 ? make_float2(0.f, 0.f) : lds_read<float2>(rec_bytes + off_colour + g * kGroupRec * 4);
+            r.colour = lds_read<float2>(rec_bytes + off_colour + g * kGroupRec * 4);
             return r;
         };
         uint32_t packed[kSub][4][2];        // f16 weights of the group's Gaussians 0-1 and 2-3, per pixel
         float w0[kSub][4], w1[kSub][4];
-        auto shade = [&](const Staged& r, float cy, float (&w)[kSub][4], const float4& rgb) {
+        auto shade = [&](const Staged& r, float cy, float (&w)[kSub][4]) {
 #pragma unroll
-            for (int s = 0; s < kSub; s++) {
-                if (kFp32) shade_quad_fp32(quad[s], role.xy[s], r.f[s % SX], r.g[s / SX], cy, rgb);
-                else shade_quad(quad[s], role.xy[s], r.f[s % SX], r.g[s / SX], cy, w[s]);
-            }
-        };
-        // fp32 colours of Gaussian k of group g (the same address in every lane)
-        auto fetch_rgb = [&](int g, int k) {
-            return kFp32 ? lds_read<float4>(rec_bytes + off_cy + g * kGroupRec * 4 + 48 + 16 * k) : make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int s = 0; s < kSub; s++) shade_quad(quad[s], role.xy[s], r.f[s % SX], r.g[s / SX], cy, w[s]);
         };
         auto pack = [&](int half) {
-            if (kFp32) return;
 #pragma unroll
             for (int s = 0; s < kSub; s++)
 #pragma unroll
                 for (int p = 0; p < 4; p++) packed[s][p][half] = pack_f16(w0[s][p], w1[s][p]);
         };
         auto accumulate = [&](const StagedGroup& grp) {
-            if (kFp32) return;
             const half4_t colour = __builtin_bit_cast(half4_t, grp.colour);
 #pragma unroll
             for (int s = 0; s < kSub; s++)
@@ -490,19 +476,17 @@ __device__ __forceinline__ bool walk_list(
         if (4 * (G) >= cnt) break;                                                           \
         grp = next_grp;                                                                      \
         next_grp = fetch_group(((G) + 1) % kGroups);    /* past the batch: read and dropped */\
-        rgb0 = fetch_rgb(G, 0); rgb1 = fetch_rgb(G, 1);                                      \
         second = fetch(4 * (G) + 1);                                                         \
-        shade(first, grp.cy.x, w0, rgb0);                                                    \
+        shade(first, grp.cy.x, w0);                                                          \
         first = fetch(4 * (G) + 2);                                                          \
-        shade(second, grp.cy.y, w1, rgb1);                                                   \
+        shade(second, grp.cy.y, w1);                                                         \
         pack(0);                                                                             \
         stop_mid = all_stopped();                                                            \
         if (!stop_mid) {                                                                     \
-            rgb0 = fetch_rgb(G, 2); rgb1 = fetch_rgb(G, 3);                                  \
             second = fetch(4 * (G) + 3);                                                     \
-            shade(first, grp.cy.z, w0, rgb0);                                                \
+            shade(first, grp.cy.z, w0);                                                      \
             first = fetch((4 * (G) + 4) % kBatch);                                           \
-            shade(second, grp.cy.w, w1, rgb1);                                               \
+            shade(second, grp.cy.w, w1);                                                     \
             pack(1);                                                                         \
         } else {                                                                             \
             _Pragma("unroll") for (int s = 0; s < kSub; s++)                                 \
@@ -513,7 +497,6 @@ __device__ __forceinline__ bool walk_list(
         static_assert(kBatch == 32, "the groups below cover a batch of 32");
         Staged first = fetch(0), second;
         StagedGroup grp, next_grp = fetch_group(0);
-        float4 rgb0, rgb1;
         bool stop_mid = false;
         do {
             FGS_GROUP(0) FGS_GROUP(1) FGS_GROUP(2) FGS_GROUP(3) FGS_GROUP(4) FGS_GROUP(5) FGS_GROUP(6) FGS_GROUP(7)
@@ -527,7 +510,7 @@ __device__ __forceinline__ bool walk_list(
     static_assert(Role::kStage >= 16 * 68, "the staging area holds the 64 x 16 colour sums of a sub-tile");
     const int lane = lane_id();
 #pragma unroll
-    for (int s = 0; s < (kFp32 ? 0 : kSub); s++) {
+    for (int s = 0; s < kSub; s++) {
         __builtin_amdgcn_wave_barrier();
         char* const out = reinterpret_cast<char*>(s_rec) + 4 * ((lane >> 2) * 68 + (lane & 3));
 #pragma unroll
@@ -546,6 +529,133 @@ __device__ __forceinline__ bool walk_list(
     }
     __builtin_amdgcn_wave_barrier();
     return done;
+}
+
+// The same walk with every operation in fp32 (render.cu:40-52 operation for operation): the colour
+// sums are three multiply-adds per pixel, and a staged Gaussian is one record - F table, G table,
+// (cy, red, green, blue) - so a lane reads all it needs of a Gaussian with three LDS reads and
+// nothing is converted, packed or handed between lanes.  Same arguments and result as walk_list.
+template <int SX, int SY>
+__device__ __forceinline__ bool walk_list_fp32(
+    const LaneRole<SX, SY>& role, float* s_rec,
+    const uint32_t* __restrict__ point_list, int begin, int n,
+    float centre_x, float centre_y,
+    const float2* __restrict__ points_xy,
+    const float4* __restrict__ rgb_depth,
+    const float4* __restrict__ conic_opacity,
+    Quad (&quad)[SX * SY])
+{
+    constexpr int kSub = SX * SY;
+    constexpr int kFx = 16 * SX, kGy = 16 * SY;
+    constexpr int kTab = kFx > kGy ? kFx : kGy;
+    constexpr int kRec = LaneRole<SX, SY>::kRec;        // kFx + kGy + 4: the tables, then (cy, r, g, b)
+    struct Staged {
+        float4 u;
+        float2 f[SX], g[SY];
+    };
+    const char* const rec_bytes = reinterpret_cast<const char*>(s_rec);
+    const uint32_t off_f = role.off_f, off_g = role.off_g;
+    uint32_t off_u = 4u * (uint32_t)(kFx + kGy);
+    asm volatile("" : "+v"(off_u));                     // kept in a vector register: reads are "register + immediate"
+    const int stage_slot = role.stage_slot;
+    const bool stage_g = role.stage_g;
+    float* const stage_tab = s_rec + stage_slot * kRec + (stage_g ? kFx : 0);
+    const int stage_len = stage_g ? kGy : kFx;
+    const int last = begin + n - 1;
+
+#pragma unroll
+    for (int s = 0; s < kSub; s++) clear_quad(quad[s]);
+
+    // registers hold the batch that is staged next; the list index is fetched two batches ahead
+    // and the attributes one batch ahead (see walk_list)
+    float2 nxy = make_float2(0.f, 0.f);
+    float4 nco = make_float4(0.f, 0.f, 0.f, 0.f), nrgb = make_float4(0.f, 0.f, 0.f, 0.f);
+    uint32_t g_ahead = 0;
+    if (n > 0) {
+        const uint32_t g = point_list[min(begin + stage_slot, last)];
+        g_ahead = point_list[min(begin + kBatch + stage_slot, last)];
+        nxy = points_xy[g]; nco = conic_opacity[g]; nrgb = rgb_depth[g];
+    }
+
+    bool done = false;
+    for (int base = 0; base < n && !done; base += kBatch) {
+        const int cnt = min(kBatch, n - base);
+        __builtin_amdgcn_wave_barrier();
+        {
+            // the entry for column (row) k is con + d (curv d + lin) at d = e - k, as a polynomial in k
+            const float ex = nxy.x - centre_x, ey = nxy.y - centre_y;
+            const float e = stage_g ? ey + (float)(kGy / 2) : ex + (float)(kFx / 2);
+            const float curv = stage_g ? nco.z : nco.x;
+            const float lin = nco.y * (stage_g ? ex : ey);
+            const float con = stage_g ? 0.0f : nco.w - (nco.y * ex) * ey;
+            const float c0 = con + e * (curv * e + lin);
+            const float c1 = -(2.0f * curv * e + lin);
+#pragma unroll
+            for (int k = 0; k < kTab; k += 4) {
+                float4 t;
+                float* tv = &t.x;
+#pragma unroll
+                for (int c = 0; c < 4; c++) tv[c] = c0 + (float)(k + c) * (c1 + curv * (float)(k + c));
+                if (k < stage_len) *reinterpret_cast<float4*>(stage_tab + k) = t;
+            }
+            if (stage_g) *reinterpret_cast<float4*>(s_rec + stage_slot * kRec + kFx + kGy) =
+                make_float4(nco.y, nrgb.x, nrgb.y, nrgb.z);
+        }
+        __builtin_amdgcn_wave_barrier();
+        nxy = points_xy[g_ahead]; nco = conic_opacity[g_ahead]; nrgb = rgb_depth[g_ahead];
+        g_ahead = point_list[min(begin + base + 2 * kBatch + stage_slot, last)];
+        // the reads of a Gaussian are issued before the Gaussian ahead of it is shaded
+        auto fetch = [&](int j) {
+            const int rec = j * kRec * 4;
+            Staged r;
+            r.u = lds_read<float4>(rec_bytes + off_u + rec);
+#pragma unroll
+            for (int c = 0; c < SX; c++) r.f[c] = lds_read<float2>(rec_bytes + off_f + rec + c * 64);
+#pragma unroll
+            for (int c = 0; c < SY; c++) r.g[c] = lds_read<float2>(rec_bytes + off_g + rec + c * 64);
+            return r;
+        };
+        auto shade = [&](const Staged& r) {
+#pragma unroll
+            for (int s = 0; s < kSub; s++)
+                shade_quad_fp32(quad[s], role.xy[s], r.f[s % SX], r.g[s / SX], r.u.x, make_float4(r.u.y, r.u.z, r.u.w, 0.f));
+        };
+        auto all_stopped = [&]() {
+            float live = quad[0].T[1][1];           // the largest T of this lane's pixels
+#pragma unroll
+            for (int s = 0; s < kSub; s++) {
+                live = __builtin_fmaxf(__builtin_fmaxf(live, quad[s].T[0][0]), __builtin_fmaxf(quad[s].T[0][1], quad[s].T[1][0]));
+                if (s > 0) live = __builtin_fmaxf(live, quad[s].T[1][1]);
+            }
+            return ballot(!(live < 0.0001f)) == 0;
+        };
+        // Gaussians go in pairs, the tile-wide stop is tested after each pair (render.cu:394-408);
+        // written out for the whole batch so that every record offset is an immediate
+#define FGS_PAIR(J)                                                                   \
+        if ((J) >= cnt) break;                                                        \
+        second = fetch((J) + 1);                                                      \
+        shade(first);                                                                 \
+        if ((J) + 1 >= cnt) break;              /* odd tail (render.cu:486-487) */    \
+        first = fetch(((J) + 2) % kBatch);      /* past the batch: read and dropped */\
+        shade(second);                                                                \
+        if (all_stopped()) { done = true; break; }
+        static_assert(kBatch == 32, "the pairs below cover a batch of 32");
+        Staged first = fetch(0), second;
+        do {
+            FGS_PAIR(0) FGS_PAIR(2) FGS_PAIR(4) FGS_PAIR(6) FGS_PAIR(8) FGS_PAIR(10) FGS_PAIR(12) FGS_PAIR(14)
+            FGS_PAIR(16) FGS_PAIR(18) FGS_PAIR(20) FGS_PAIR(22) FGS_PAIR(24) FGS_PAIR(26) FGS_PAIR(28) FGS_PAIR(30)
+        } while (0);
+#undef FGS_PAIR
+    }
+    __builtin_amdgcn_wave_barrier();
+    return done;
+}
+
+template <int SX, int SY, bool kFp32, typename... Args>
+__device__ __forceinline__ bool walk(Args&&... args)
+{
+    if constexpr (kFp32) return walk_list_fp32<SX, SY>(args...);
+    else return walk_list<SX, SY>(args...);
 }
 
 // render.cu:59-73
@@ -630,7 +740,7 @@ __device__ __forceinline__ void blend_tile(
 #pragma unroll
     for (int s = 0; s < kSub; s++) clear_quad(quad[s]);
     const float centre_x = (float)(tile_x * kFx + kFx / 2), centre_y = (float)(tile_y * kGy + kGy / 2);
-    walk_list<SX, SY, kFp32>(role, s_rec, point_list, range.x, n, centre_x, centre_y, points_xy, rgb_depth, conic_opacity, quad);
+    walk<SX, SY, kFp32>(role, s_rec, point_list, range.x, n, centre_x, centre_y, points_xy, rgb_depth, conic_opacity, quad);
     write_tile<SX, SY>(lane, tile_x, tile_y, width, height, quad, bg_r, bg_g, bg_b, out_u8, out_f32);
 }
 
@@ -732,7 +842,7 @@ __global__ __launch_bounds__(kSharedWaves * kWave) __attribute__((amdgpu_waves_p
             count = min(run, rest - skip);
         }
         clear_quad(part[0]);
-        const bool stopped = walk_list<1, 1, kFp32>(role, s_rec[wave], point_list, __builtin_amdgcn_readfirstlane(s_from[v]) + skip, count,
+        const bool stopped = walk<1, 1, kFp32>(role, s_rec[wave], point_list, __builtin_amdgcn_readfirstlane(s_from[v]) + skip, count,
                                              (float)(__builtin_amdgcn_readfirstlane(s_tile_x[v]) * 16 + 8),
                                              (float)(__builtin_amdgcn_readfirstlane(s_tile_y[v]) * 16 + 8),
                                              points_xy, rgb_depth, conic_opacity, part);

@@ -995,6 +995,11 @@ __global__ __launch_bounds__(kWave) void segment_sort_wave_list_kernel(
 // The same passes with whole keys and the ping-pong copy in HBM: for segments longer than
 // min_len and for shorter segments whose keys differ above the depth word.  General and slow;
 // inputs produced by fgs_preprocess only reach it with more than min_len pairs in one tile.
+// Sixteen waves per workgroup: such a segment has thousands of pairs, every pass reads them from
+// memory 64 per wave and step, and the workgroup has the CU almost to itself (a frame of 109M
+// pairs with 534 such segments: 0.55 ms for the launch with four waves).
+constexpr int kGeneralWaves = 16;
+
 __device__ __forceinline__ void sort_segment_general(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
                                                      uint64_t* __restrict__ alt_keys, uint32_t* __restrict__ alt_values,
                                                      int lo, int hi, uint32_t (*s_cnt)[kBins], uint32_t* s_wave_sum, int* s_flag)
@@ -1006,14 +1011,14 @@ __device__ __forceinline__ void sort_segment_general(uint64_t* __restrict__ keys
     int cur = 0;
 #pragma unroll 1
     for (int shift = 0; shift < 32; shift += 8) {
-        const bool moved = counting_pass<kSortWaves, uint64_t>(kbuf[cur], vbuf[cur], kbuf[cur ^ 1], vbuf[cur ^ 1], len,
-                                                               shift, s_cnt, s_wave_sum, s_flag);
+        const bool moved = counting_pass<kGeneralWaves, uint64_t>(kbuf[cur], vbuf[cur], kbuf[cur ^ 1], vbuf[cur ^ 1], len,
+                                                                  shift, s_cnt, s_wave_sum, s_flag);
         __threadfence_block();
         __syncthreads();
         if (moved) cur ^= 1;
     }
     if (cur == 1)
-        for (int i = tid; i < len; i += kSortBlock) { kbuf[0][i] = kbuf[1][i]; vbuf[0][i] = vbuf[1][i]; }
+        for (int i = tid; i < len; i += kGeneralWaves * kWave) { kbuf[0][i] = kbuf[1][i]; vbuf[0][i] = vbuf[1][i]; }
     __threadfence_block();
     __syncthreads();
 }
@@ -1022,15 +1027,15 @@ __device__ __forceinline__ void sort_segment_general(uint64_t* __restrict__ keys
 // ones longer than min_len: neighbouring tiles tend to be equally crowded, so they are dealt out
 // one segment at a time, round-robin), the workgroups behind them look at 64 tile ids each for
 // shorter segments that were flagged.
-__global__ __launch_bounds__(kSortBlock) void segment_sort_general_kernel(
+__global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_kernel(
     uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
     uint64_t* __restrict__ alt_keys, uint32_t* __restrict__ alt_values,
     int n, uint32_t tile_mask, int min_len, uint32_t ids,
     const int* __restrict__ seg_start, const uint32_t* __restrict__ seg_flags,
     const uint32_t* __restrict__ list, const uint32_t* __restrict__ list_count, uint32_t list_cap, uint32_t list_blocks)
 {
-    __shared__ uint32_t s_cnt[kSortWaves][kBins];
-    __shared__ uint32_t s_wave_sum[kSortWaves];
+    __shared__ uint32_t s_cnt[kGeneralWaves][kBins];
+    __shared__ uint32_t s_wave_sum[kGeneralWaves];
     __shared__ int s_bounds[2];
     __shared__ int s_flag;
     __shared__ uint64_t s_match;
@@ -1052,7 +1057,7 @@ __global__ __launch_bounds__(kSortBlock) void segment_sort_general_kernel(
         if (len <= min_len) {       // without flags the shorter segments are re-examined here
             const uint32_t upper = (uint32_t)(keys[lo] >> 32);
             bool mixed = false;
-            for (int i = tid; i < len; i += kSortBlock) mixed = mixed || (uint32_t)(keys[lo + i] >> 32) != upper;
+            for (int i = tid; i < len; i += kGeneralWaves * kWave) mixed = mixed || (uint32_t)(keys[lo + i] >> 32) != upper;
             if (mixed) s_flag = 1;
             __syncthreads();
             const bool any_mixed = s_flag != 0;
@@ -1262,7 +1267,7 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         // longer segments from their list, one workgroup per segment; behind them the shorter ones that were flagged
         const unsigned long_blocks = seg_start && n > kCapLarge ? list_grid((unsigned)(n / (kCapLarge + 1) + 1), 2048u) : 0u;
         hipLaunchKernelGGL(segment_sort_general_kernel, dim3(seg_start ? long_blocks + (ids + kWave - 1) / kWave : ids),
-                           dim3(kSortBlock), 0, st, ks, vs, alt_keys, alt_values, n, tile_mask, kCapLarge, ids,
+                           dim3(kGeneralWaves * kWave), 0, st, ks, vs, alt_keys, alt_values, n, tile_mask, kCapLarge, ids,
                            (const int*)seg_start, (const uint32_t*)seg_flags,
                            (const uint32_t*)list_long, (const uint32_t*)(seg_counts + 3 * kListShards), cap_long, long_blocks);
     }

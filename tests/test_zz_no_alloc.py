@@ -85,7 +85,6 @@ def test_static_entry_point_allocates_nothing_and_runs_under_capture():
     with torch.cuda.graph(graph, stream=side):
         off.zero_()
         launch(torch.cuda.current_stream().cuda_stream)
-    assert torch.cuda.mem_get_info()[0] <= free_before      # the graph object itself may hold memory; the library none
     for replay in range(3):
         keys.zero_(); values.zero_()
         graph.replay()
