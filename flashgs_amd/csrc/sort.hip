@@ -54,6 +54,11 @@ using Narrow = PassShape<8, 16>;
 using Wide = PassShape<9, 15>;
 constexpr int kNarrowMaxTileBits = 16;
 
+
+// A list of at most kSmallRows blocks needs no launch that turns the histogram rows into starts:
+// the scatter workgroups add the rows up themselves.
+constexpr int kSmallRows = 64;
+
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 // Tile ids up to this count get a table of segment starts in the workspace; beyond it every
@@ -270,8 +275,6 @@ __global__ __launch_bounds__(kOffsetThreads) void offsets_kernel(uint32_t* __res
     }
 }
 
-// A list of at most kSmallRows histogram rows needs neither: the scatter workgroups add the rows up themselves.
-constexpr int kSmallRows = 64;
 
 // ---- step 3: stable scatter ---------------------------------------------------------------------------
 
@@ -507,6 +510,9 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
 
 // ---- per-tile segment sort on the 32 depth bits ----------------------------------------------------
 
+// size classes of the segments: pairs per segment
+constexpr int kCapTiny = 512, kCapSmall = 1024, kCapMedium = 4096, kCapLarge = 8192;
+
 // First index in [0, n) whose tile field is >= v (n if none), found by the whole wave probing 64
 // evenly spaced positions per step.  `keys` is ordered by tile field.  All lanes return the same.
 __device__ __forceinline__ int wave_lower_bound(const uint64_t* __restrict__ keys, int n, uint32_t v, uint32_t tile_mask)
@@ -675,8 +681,9 @@ __device__ __forceinline__ bool counting_pass(const KeyT* src_k, const uint32_t*
 // with the same arguments; hi - lo <= kCap.  A segment whose keys differ above the depth word
 // cannot be rebuilt from depth words: it is flagged (or, without a flag array, left alone) for
 // the general kernel.
+// Returns true when that was the case (nothing is moved then).
 template <int kWaves, int kCap>
-__device__ __forceinline__ void sort_segment_lds(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
+__device__ __forceinline__ bool sort_segment_lds(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
                                                  uint32_t v, int lo, int hi, uint32_t* __restrict__ seg_flags,
                                                  uint32_t (*s_k)[kCap], uint32_t (*s_v)[kCap],
                                                  uint32_t (*s_cnt)[kBins], uint32_t* s_wave_sum, int* s_flag)
@@ -696,7 +703,7 @@ __device__ __forceinline__ void sort_segment_lds(uint64_t* __restrict__ keys, ui
     if (kWaves == 1) {
         if (ballot(mixed)) {
             if (seg_flags && lane == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
-            return;
+            return true;
         }
         __builtin_amdgcn_wave_barrier();
     } else {
@@ -706,7 +713,7 @@ __device__ __forceinline__ void sort_segment_lds(uint64_t* __restrict__ keys, ui
         __syncthreads();                             // counting_pass reuses the flag
         if (any_mixed) {
             if (seg_flags && tid == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
-            return;
+            return true;
         }
     }
 
@@ -723,6 +730,7 @@ __device__ __forceinline__ void sort_segment_lds(uint64_t* __restrict__ keys, ui
         values[lo + i] = s_v[cur][i];
     }
     if (kWaves > 1) __syncthreads(); else __builtin_amdgcn_wave_barrier();
+    return false;
 }
 
 // Segment sort in LDS for one size class: segments with min_len < length <= kCap.
@@ -1027,13 +1035,22 @@ __device__ __forceinline__ void sort_segment_general(uint64_t* __restrict__ keys
 // ones longer than min_len: neighbouring tiles tend to be equally crowded, so they are dealt out
 // one segment at a time, round-robin), the workgroups behind them look at 64 tile ids each for
 // shorter segments that were flagged.
+// With kAllClasses the listed blocks first sort the listed segments of the two classes below
+// (1025 .. kCapLarge pairs, in LDS like segment_sort_kernel<16, kCapLarge>), shard by shard like
+// the launches of those classes: a frame with a short list of pairs has few such segments or
+// none, and one launch instead of three is what counts there.
+template <bool kAllClasses>
 __global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_kernel(
     uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
     uint64_t* __restrict__ alt_keys, uint32_t* __restrict__ alt_values,
     int n, uint32_t tile_mask, int min_len, uint32_t ids,
     const int* __restrict__ seg_start, const uint32_t* __restrict__ seg_flags,
-    const uint32_t* __restrict__ list, const uint32_t* __restrict__ list_count, uint32_t list_cap, uint32_t list_blocks)
+    const uint32_t* __restrict__ list, const uint32_t* __restrict__ list_count, uint32_t list_cap, uint32_t list_blocks,
+    const uint32_t* __restrict__ list_medium, uint32_t cap_medium, const uint32_t* __restrict__ list_large, uint32_t cap_large)
 {
+    constexpr int kLdsCap = kAllClasses ? kCapLarge : 1;
+    __shared__ uint32_t s_k[2][kLdsCap];
+    __shared__ uint32_t s_v[2][kLdsCap];
     __shared__ uint32_t s_cnt[kGeneralWaves][kBins];
     __shared__ uint32_t s_wave_sum[kGeneralWaves];
     __shared__ int s_bounds[2];
@@ -1070,7 +1087,23 @@ __global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_ke
 
     if (blockIdx.x < list_blocks) {
         const uint32_t shard = blockIdx.x % kListShards;
-        const uint32_t count = list_count[shard];
+        if constexpr (kAllClasses) {
+            // list_count: the counters of all classes, class c at c * kListShards (1: medium, 2: large, 3: long)
+            for (int c = 1; c <= 2; c++) {
+                const uint32_t* const ids_of = c == 1 ? list_medium : list_large;
+                const uint32_t cap = c == 1 ? cap_medium : cap_large;
+                const uint32_t count = list_count[c * kListShards + shard];
+                for (uint32_t i = blockIdx.x / kListShards; i < count; i += list_blocks / kListShards) {
+                    const uint32_t v = ids_of[(size_t)shard * cap + i];
+                    // keys that differ above the depth word: through memory right away (no flag: the
+                    // workgroups that look at the flags run beside this one)
+                    if (sort_segment_lds<kGeneralWaves, kCapLarge>(keys, values, v, seg_start[v], seg_start[v + 1], nullptr,
+                                                                   s_k, s_v, s_cnt, s_wave_sum, &s_flag))
+                        sort_segment_general(keys, values, alt_keys, alt_values, seg_start[v], seg_start[v + 1], s_cnt, s_wave_sum, &s_flag);
+                }
+            }
+        }
+        const uint32_t count = list_count[(kAllClasses ? 3 * kListShards : 0) + shard];
         for (uint32_t i = blockIdx.x / kListShards; i < count; i += list_blocks / kListShards) {
             const uint32_t v = list[(size_t)shard * list_cap + i];
             sort_segment_general(keys, values, alt_keys, alt_values, seg_start[v], seg_start[v + 1], s_cnt, s_wave_sum, &s_flag);
@@ -1095,7 +1128,7 @@ __global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_ke
     }
 }
 
-constexpr int kCapTiny = 512, kCapSmall = 1024, kCapMedium = 4096, kCapLarge = 8192;
+constexpr int kMergedTailMax = 1 << 19;      // up to this many pairs the last launch also takes the classes of 1025 .. 8192 pairs
 constexpr uint32_t kOneLaunchIds = 32768;    // up to this many tile ids one launch sorts every segment of up to kCapSmall pairs
 
 
@@ -1245,13 +1278,16 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
                                0, st, ks, vs, n, tile_mask, 1, ids, (const int*)seg_start, seg_flags,
                                kCapSmall, kCapMedium, kCapLarge, seg_counts, seg_start ? list_small : nullptr, list_medium,
                                list_large, list_long, cap_small, cap_medium, cap_large, cap_long);
+        // A short list of pairs has few segments of more than 1024 pairs, or none: there the one
+        // launch below takes those classes too (720p, 0.2M pairs: two launches less).
+        const bool merged_tail = seg_start && n <= kMergedTailMax;
         if (seg_start) {
             if (n > kCapTiny && !one_wave_launch)       // 513..1024: the same network over 16 register slots, from the lists
                 hipLaunchKernelGGL((segment_sort_wave_list_kernel<kCapSmall / kWave>),
                                    dim3(list_grid((unsigned)(n / (kCapTiny + 1) + 1), 8192u)),
                                    dim3(kWave), 0, st, ks, vs, (const int*)seg_start, seg_flags,
                                    (const uint32_t*)list_small, (const uint32_t*)seg_counts, cap_small);
-            if (n > kCapSmall) {
+            if (n > kCapSmall && !merged_tail) {
                 FGS_SEGMENT_CLASS(8, kCapMedium, 64, kCapSmall, list_grid((unsigned)(n / (kCapSmall + 1) + 1), 1024u),
                                   list_medium, seg_counts + kListShards, cap_medium);
                 if (n > kCapMedium)
@@ -1265,11 +1301,21 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         }
 #undef FGS_SEGMENT_CLASS
         // longer segments from their list, one workgroup per segment; behind them the shorter ones that were flagged
-        const unsigned long_blocks = seg_start && n > kCapLarge ? list_grid((unsigned)(n / (kCapLarge + 1) + 1), 2048u) : 0u;
-        hipLaunchKernelGGL(segment_sort_general_kernel, dim3(seg_start ? long_blocks + (ids + kWave - 1) / kWave : ids),
-                           dim3(kGeneralWaves * kWave), 0, st, ks, vs, alt_keys, alt_values, n, tile_mask, kCapLarge, ids,
-                           (const int*)seg_start, (const uint32_t*)seg_flags,
-                           (const uint32_t*)list_long, (const uint32_t*)(seg_counts + 3 * kListShards), cap_long, long_blocks);
+        if (merged_tail) {
+            const unsigned blocks = n > kCapSmall ? list_grid((unsigned)(n / (kCapSmall + 1) + 1), 256u) : 0u;
+            hipLaunchKernelGGL(segment_sort_general_kernel<true>, dim3(blocks + (ids + kWave - 1) / kWave),
+                               dim3(kGeneralWaves * kWave), 0, st, ks, vs, alt_keys, alt_values, n, tile_mask, kCapLarge, ids,
+                               (const int*)seg_start, (const uint32_t*)seg_flags,
+                               (const uint32_t*)list_long, (const uint32_t*)seg_counts, cap_long, blocks,
+                               (const uint32_t*)list_medium, cap_medium, (const uint32_t*)list_large, cap_large);
+        } else {
+            const unsigned long_blocks = seg_start && n > kCapLarge ? list_grid((unsigned)(n / (kCapLarge + 1) + 1), 2048u) : 0u;
+            hipLaunchKernelGGL(segment_sort_general_kernel<false>, dim3(seg_start ? long_blocks + (ids + kWave - 1) / kWave : ids),
+                               dim3(kGeneralWaves * kWave), 0, st, ks, vs, alt_keys, alt_values, n, tile_mask, kCapLarge, ids,
+                               (const int*)seg_start, (const uint32_t*)seg_flags,
+                               (const uint32_t*)list_long, (const uint32_t*)(seg_counts + 3 * kListShards), cap_long, long_blocks,
+                               no_list, 0u, no_list, 0u);
+        }
     }
     return check_hip(hipGetLastError(), "sort launch");
 }
