@@ -34,8 +34,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3         # MI355X fp32 vector, published (packed FMA)
 FLOP_PER_EVAL = 19               # render.cu:40-52: 2 sub, 6 mul + 3 add, 1 mul, 3 FMA, 1 sub
-EXEC_SLOTS_PER_EVAL = 9          # what the fp32 blend kernel issues: 2 for the exponent from its tables, exp2 at half
-                                 # rate = 2, alpha*T, T -= , 3 colour FMAs
+EXEC_SLOTS_PER_EVAL = 8.1        # non-transcendental VALU instructions the fp32 blend kernel issues per evaluation (SQ counters,
+                                 # profiles/frame_cfg2_3M_4K_sq_counters.txt): 2 for the exponent from its tables, alpha*T, T -=,
+                                 # 3 colour FMAs, 1.1 for staging, stop tests and loop; the v_exp_f32 issues beside them
 ATTAINED_FMA_LANE_OPS = 38.05e12 # v_fma_f32 lane-operations/s measured on this part without packed math (bench.py --calibrate)
 CAPACITY = {0: 1 << 20, 1: 1 << 22, 2: 1 << 24, 3: 1 << 25, 4: 1 << 25, 5: 1 << 27}
 FAST_MODE_DTYPE = "f32 (colour sums: f16 operands on the matrix unit, fp32 products and sums)"
@@ -269,12 +270,12 @@ def stage_report(fr, stage_ms, K, counts, walked):
         # reference-equivalent work: the 19 flop of render.cu:40-52 per pixel-Gaussian evaluation over the
         # published fp32 vector peak (which counts packed FMA; this library issues none)
         tflops = FLOP_PER_EVAL * evals / (blend_ms * 1e-3) / 1e12
-        # executed work: the kernel's own 9 issue slots per evaluation over the v_fma_f32 rate this part attains
+        # executed work: the kernel's own VALU instructions per evaluation over the v_fma_f32 rate this part attains
         floor_ms = EXEC_SLOTS_PER_EVAL * evals / ATTAINED_FMA_LANE_OPS * 1e3
         roofline.update(achieved=round(tflops, 2), frac=round(tflops / FP32_PEAK_TFLOPS, 4),
                         achieved_is="reference-equivalent flop (19 per evaluation, render.cu:40-52) per second",
                         evaluations=int(evals), flop_per_evaluation=FLOP_PER_EVAL,
-                        executed_issue_slots_per_evaluation=EXEC_SLOTS_PER_EVAL,
+                        executed_valu_instructions_per_evaluation=EXEC_SLOTS_PER_EVAL,
                         issue_bound_ms=round(floor_ms, 4), frac_of_attained_issue_rate=round(floor_ms / blend_ms, 4),
                         hbm_bytes=int(8 * tiles + 44 * walked + 3 * W * H))
         stages["blend"].update(achieved_TFLOPs=roofline["achieved"], frac=roofline["frac"])
@@ -298,6 +299,8 @@ def ops_surface_ms(torch, np, fr, steps):
         img = rast.forward(scene, cam, bg)
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / steps
+    fr.frame(fr.cams[0])                        # the same frame through the C ABI, library default like the ops
+    torch.cuda.synchronize()
     same = bool(torch.equal(img, fr.out_color))
     del rast
     return round(ms, 4), same
