@@ -10,9 +10,11 @@
 // batch are already in flight; the wave then walks the batch, every lane reading the table
 // entries of its own columns and rows.  After every second Gaussian one ballot tests whether all
 // pixels of the tile have T < 1e-4, which is the reference's stop rule (render.cu:394-408).  A
-// workgroup is a single wave, so no workgroup barrier is needed anywhere.  The colour sums go
-// through the matrix unit four Gaussians at a time (f16 operands, fp32 accumulation) or, on
-// request (fgs_set_colour_sums), through fp32 multiply-adds; every kernel exists in both forms.
+// workgroup is a single wave, so no workgroup barrier is needed anywhere.  Every kernel exists in
+// two forms: all fp32, operation for operation the reference's pixel shader (the default), and
+// with the colour sums on the matrix unit four Gaussians at a time (f16 operands, fp32
+// accumulation), which a caller asks for per call (FGS_BLEND_MATRIX_F16) or per process
+// (fgs_set_colour_sums).
 #include "fgs_internal.h"
 
 #include <atomic>

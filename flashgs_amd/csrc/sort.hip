@@ -18,11 +18,11 @@
 //     last scatter pass also tabulates where each tile id's segment begins (with more than two
 //     passes `segment_starts_kernel` does, from the sorted keys), then segments are handled by
 //     size class.  Up to 1024 pairs one wave holds the segment in registers as 64-bit
-//     words depth << 32 | position and runs a bitonic network on them (all words differ, so the
-//     result is that of a stable sort by depth); lane exchanges inside a row of 16 lanes are
+//     words depth << 32 | value (| position where the values of a segment do not ascend) and runs
+//     a bitonic network on them (the result is that of a stable sort by depth); lane exchanges inside a row of 16 lanes are
 //     data-parallel-primitive moves.  Up to 4096 (8 waves) and 8192 pairs (16 waves) a workgroup
-//     runs up to four stable 8-bit counting passes in LDS, skipping a pass in which all pairs
-//     share the digit.  Longer segments, and segments whose keys differ above the sorted bit
+//     runs up to four stable 8-bit counting passes in LDS (in place: the pairs wait in registers
+//     while they are counted), skipping a pass in which all pairs share the digit.  Longer segments, and segments whose keys differ above the sorted bit
 //     range, go through the same passes with the ping-pong copy in HBM instead of LDS.
 //
 // Bytes moved per pair: 8 (count) + 24 (scatter) per partition pass, 24 for the segment sort:
@@ -512,6 +512,8 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
 
 // size classes of the segments: pairs per segment
 constexpr int kCapTiny = 512, kCapSmall = 1024, kCapMedium = 4096, kCapLarge = 8192;
+constexpr int kMergedTailMax = 1 << 19;      // up to this many pairs the last launch also takes the classes of 1025 .. 8192 pairs
+constexpr uint32_t kOneLaunchIds = 32768;    // up to this many tile ids one launch sorts every segment of up to kCapSmall pairs
 
 // First index in [0, n) whose tile field is >= v (n if none), found by the whole wave probing 64
 // evenly spaced positions per step.  `keys` is ordered by tile field.  All lanes return the same.
@@ -543,10 +545,11 @@ constexpr int kStartsPerThread = 8;
 
 __global__ __launch_bounds__(256) void segment_starts_kernel(const uint64_t* __restrict__ keys, int n, uint32_t tile_mask,
                                                              uint32_t ids, int* __restrict__ seg_start,
-                                                             uint32_t* __restrict__ seg_flags, uint32_t* __restrict__ seg_counts)
+                                                             uint32_t* __restrict__ seg_flags, uint32_t flag_words,
+                                                             uint32_t* __restrict__ seg_counts)
 {
     const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
-    for (uint32_t w = gid; w < (ids + 31) / 32; w += gridDim.x * blockDim.x) seg_flags[w] = 0;
+    for (uint32_t w = gid; w < flag_words; w += gridDim.x * blockDim.x) seg_flags[w] = 0;
     if (gid < (uint32_t)(kListClasses * kListShards)) seg_counts[gid] = 0;
     const long long base = (long long)blockIdx.x * (256 * kStartsPerThread) + threadIdx.x;
     uint32_t cur[kStartsPerThread], before[kStartsPerThread];
@@ -677,6 +680,93 @@ __device__ __forceinline__ bool counting_pass(const KeyT* src_k, const uint32_t*
     return true;
 }
 
+// The same pass over a segment of depth words and values held in LDS, in place: every thread takes
+// its kPer pairs into registers (pair w_lo + it*64 + lane for it < kPer, so a wave still ranks its
+// contiguous part 64 pairs at a time in segment order), and once all of them are counted nobody
+// needs the arrays any more and the ranked pairs go back into them.  Half the LDS of a ping-pong
+// copy, and one read of every pair instead of two.  The counters are 16 bits wide (positions stay
+// below 65536), two to a word, counted with 32-bit atomic additions on the half that is meant.
+template <int kWaves, int kPer>
+__device__ __forceinline__ bool counting_pass_lds(uint32_t* s_k, uint32_t* s_v, int n, int shift,
+                                                  uint16_t (*cnt)[kBins], uint32_t* wave_sum, int* flag)
+{
+    static_assert(kWaves * kWave >= kBins, "one thread per digit in the scan");
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+    const int per = ((n + kWaves - 1) / kWaves + kWave - 1) / kWave * kWave;   // a multiple of 64, at most 64 * kPer
+    const int w_lo = min(n, wave * per), w_hi = min(n, w_lo + per);
+
+    uint32_t* const cnt_words = (uint32_t*)cnt[wave];
+    cnt_words[lane] = 0;
+    cnt_words[lane + kWave] = 0;
+    if (tid == 0) *flag = 0;
+    __syncthreads();
+    uint32_t k[kPer], v[kPer];
+#pragma unroll
+    for (int it = 0; it < kPer; it++) {
+        const int i = w_lo + it * kWave + lane;
+        k[it] = 0; v[it] = 0;
+        if (i < w_hi) {
+            k[it] = s_k[i];
+            v[it] = s_v[i];
+            const uint32_t d = (k[it] >> shift) & 255u;
+            atomicAdd(&cnt_words[d >> 1], (d & 1u) ? 0x10000u : 1u);
+        }
+    }
+    __syncthreads();
+
+    uint32_t total = 0;
+    if (tid < kBins) {                   // thread t handles digit t
+        for (int w = 0; w < kWaves; w++) {
+            const uint32_t c = cnt[w][tid];
+            cnt[w][tid] = (uint16_t)total;          // offset of wave w inside digit tid
+            total += c;
+        }
+        if (total == (uint32_t)n) *flag = 1;
+        const uint32_t incl = wave_inclusive_sum(total);
+        if (lane == kWave - 1) wave_sum[wave] = incl;
+        total = incl - total;             // exclusive inside this wave's 64 digits
+    }
+    __syncthreads();
+    if (tid < kBins) {
+        uint32_t base = total;
+        for (int w = 0; w < wave; w++) base += wave_sum[w];
+        for (int w = 0; w < kWaves; w++) cnt[w][tid] = (uint16_t)(cnt[w][tid] + base);     // absolute start of (wave, digit)
+    }
+    __syncthreads();
+    if (*flag != 0) return false;        // every pair has the same digit: nothing to move
+
+    // stable ranking, 64 pairs at a time in segment order
+#pragma unroll
+    for (int it = 0; it < kPer; it++) {
+        if (w_lo + it * kWave >= w_hi) break;
+        const bool valid = w_lo + it * kWave + lane < w_hi;
+        const uint32_t d = (k[it] >> shift) & 255u;
+        uint64_t peers = ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            const bool bit = (d >> b) & 1u;
+            const uint64_t with_bit = ballot(bit);
+            peers &= bit ? with_bit : ~with_bit;
+        }
+        const int below = popc_below(peers);
+        uint32_t before = 0;
+        if (valid && below == 0) {
+            before = cnt[wave][d];
+            cnt[wave][d] = (uint16_t)(before + (uint32_t)__popcll(peers));
+        }
+        const int leader = valid ? __ffsll((long long)peers) - 1 : lane;
+        before = (uint32_t)__shfl((int)before, leader);
+        if (valid) {
+            s_k[before + (uint32_t)below] = k[it];
+            s_v[before + (uint32_t)below] = v[it];
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    return true;
+}
+
 // Sorts the segment [lo, hi) of tile id v in LDS.  Called by all kWaves waves of a workgroup
 // with the same arguments; hi - lo <= kCap.  A segment whose keys differ above the depth word
 // cannot be rebuilt from depth words: it is flagged (or, without a flag array, left alone) for
@@ -685,51 +775,41 @@ __device__ __forceinline__ bool counting_pass(const KeyT* src_k, const uint32_t*
 template <int kWaves, int kCap>
 __device__ __forceinline__ bool sort_segment_lds(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
                                                  uint32_t v, int lo, int hi, uint32_t* __restrict__ seg_flags,
-                                                 uint32_t (*s_k)[kCap], uint32_t (*s_v)[kCap],
-                                                 uint32_t (*s_cnt)[kBins], uint32_t* s_wave_sum, int* s_flag)
+                                                 uint32_t* s_k, uint32_t* s_v,
+                                                 uint16_t (*s_cnt)[kBins], uint32_t* s_wave_sum, int* s_flag)
 {
+    static_assert(kCap % (kWaves * kWave) == 0, "every thread holds the same number of pairs");
     const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
     const int len = hi - lo;
     const uint32_t upper = (uint32_t)(keys[lo] >> 32);
     bool mixed = false;
-    if (kWaves > 1) { if (tid == 0) *s_flag = 0; __syncthreads(); }
+    if (tid == 0) *s_flag = 0;
+    __syncthreads();
     for (int i = tid; i < len; i += kWaves * kWave) {
         const uint64_t k = keys[lo + i];
-        s_k[0][i] = (uint32_t)k;
-        s_v[0][i] = values[lo + i];
+        s_k[i] = (uint32_t)k;
+        s_v[i] = values[lo + i];
         mixed = mixed || (uint32_t)(k >> 32) != upper;
     }
-    if (kWaves == 1) {
-        if (ballot(mixed)) {
-            if (seg_flags && lane == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
-            return true;
-        }
-        __builtin_amdgcn_wave_barrier();
-    } else {
-        if (mixed) *s_flag = 1;
-        __syncthreads();
-        const bool any_mixed = *s_flag != 0;
-        __syncthreads();                             // counting_pass reuses the flag
-        if (any_mixed) {
-            if (seg_flags && tid == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
-            return true;
-        }
+    if (mixed) *s_flag = 1;
+    __syncthreads();
+    const bool any_mixed = *s_flag != 0;
+    __syncthreads();                             // the passes reuse the flag
+    if (any_mixed) {
+        if (seg_flags && tid == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
+        return true;
     }
 
-    int cur = 0;
 #pragma unroll 1
     for (int shift = 0; shift < 32; shift += 8) {
-        const bool moved = counting_pass<kWaves, uint32_t>(s_k[cur], s_v[cur], s_k[cur ^ 1], s_v[cur ^ 1], len, shift,
-                                                           s_cnt, s_wave_sum, s_flag);
-        if (kWaves > 1) __syncthreads(); else __builtin_amdgcn_wave_barrier();
-        if (moved) cur ^= 1;
+        counting_pass_lds<kWaves, kCap / (kWaves * kWave)>(s_k, s_v, len, shift, s_cnt, s_wave_sum, s_flag);
+        __syncthreads();
     }
     for (int i = tid; i < len; i += kWaves * kWave) {
-        keys[lo + i] = ((uint64_t)upper << 32) | s_k[cur][i];
-        values[lo + i] = s_v[cur][i];
+        keys[lo + i] = ((uint64_t)upper << 32) | s_k[i];
+        values[lo + i] = s_v[i];
     }
-    if (kWaves > 1) __syncthreads(); else __builtin_amdgcn_wave_barrier();
+    __syncthreads();
     return false;
 }
 
@@ -743,9 +823,9 @@ __global__ __launch_bounds__(kWaves * kWave) void segment_sort_kernel(
     const int* __restrict__ seg_start, uint32_t* __restrict__ seg_flags,
     const uint32_t* __restrict__ list, const uint32_t* __restrict__ list_count, uint32_t list_cap)
 {
-    __shared__ uint32_t s_k[2][kCap];
-    __shared__ uint32_t s_v[2][kCap];
-    __shared__ uint32_t s_cnt[kWaves][kBins];
+    __shared__ uint32_t s_k[kCap];
+    __shared__ uint32_t s_v[kCap];
+    __shared__ __align__(4) uint16_t s_cnt[kWaves][kBins];
     __shared__ uint32_t s_wave_sum[kWaves];
     __shared__ int s_bounds[2];
     __shared__ int s_flag;
@@ -830,9 +910,12 @@ __device__ __forceinline__ void bitonic_network(uint64_t (&c)[kT], int lane)
     constexpr int n = kT * kWave;
 #pragma unroll 1
     for (int k = 2; k <= n; k <<= 1) {
-        bool ascending[kT];                 // element lane*kT + t sits in an ascending run of width k
+        // element lane*kT + t sits in an ascending run of width k: a matter of t alone while the
+        // runs are shorter than a lane's slots, of the lane alone from there on
+        bool ascending[kT];
+        const bool lane_ascending = (lane & (k / kT)) == 0;
 #pragma unroll
-        for (int t = 0; t < kT; t++) ascending[t] = ((lane * kT + t) & k) == 0;
+        for (int t = 0; t < kT; t++) ascending[t] = k < kT ? (t & k) == 0 : lane_ascending;
 #pragma unroll
         for (int j = n / 2; j > 0; j >>= 1) {
             if (j >= k) continue;
@@ -864,74 +947,120 @@ __device__ __forceinline__ void bitonic_network(uint64_t (&c)[kT], int lane)
     }
 }
 
+// Words of LDS a wave needs to sort up to n pairs with the network: one 64-bit word per pair, one
+// word of padding after every 16 (lane l puts its kUse consecutive ranks down at once; without
+// the padding the lanes of a wave would all start in the same bank).
+__host__ __device__ constexpr int staging_words(int n) { return n + n / 16; }
+__device__ __forceinline__ int staged(int i) { return i + (i >> 4); }
+
 // Sorts the segment [lo, hi) of tile id v with the network over kUse slots per lane, 64 * kUse >= hi - lo.
-// Every word carries its element's position, so it does not matter which slot an element starts
-// in: the loads are the contiguous ones (element t*64 + lane in slot t), the network leaves rank
-// lane*kUse + t in slot t, and the sorted pairs go through LDS to be stored contiguously again.
-// s_v holds three arrays of kStride words: values by position, sorted depths, sorted values.
-template <int kUse, int kStride>
+// The network orders 64-bit words, depth above and a tie-break below, and it does not matter
+// which slot a word starts in: the loads are the contiguous ones (element t*64 + lane in slot t),
+// the network leaves rank lane*kUse + t in slot t, and the sorted words go through LDS to be
+// stored contiguously again.  Equal depths have to stay in input order.  The pairs of one tile
+// come out of the preprocess in ascending order of their values (Gaussian indices): then the value
+// itself is the tie-break and the sorted word is the pair.  A segment whose values do not ascend
+// carries positions instead and looks its values up afterwards.
+template <int kUse>
 __device__ __forceinline__ void sort_segment_bitonic_of(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
                                                         uint32_t v, int lo, int hi, uint32_t* __restrict__ seg_flags,
-                                                        uint32_t* s_v)
+                                                        uint64_t* s_w)
 {
-    const int lane = threadIdx.x & (kWave - 1);
+    // The lane number is made opaque here and again behind the network: otherwise every index and
+    // address derived from it, for every width of the network, is computed once in front of the loop
+    // over the segments and kept in registers through all of it (80 registers of a 16-slot network).
+    int lane = threadIdx.x & (kWave - 1);
+    asm volatile("" : "+v"(lane));
     const int len = hi - lo;
-    const uint32_t upper = (uint32_t)(keys[lo] >> 32);
-    uint32_t* const s_depth = s_v + kStride;
-    uint32_t* const s_value = s_v + 2 * kStride;
     uint64_t c[kUse];
+    uint32_t val[kUse];
+    const uint64_t* const seg_keys = keys + lo;
+    const uint32_t* const seg_values = values + lo;
+    // Every load is issued before the first one is looked at: a slot past the end of the segment
+    // reads the last pair again (a load under a condition would be waited for before the next).
+#pragma unroll
+    for (int t = 0; t < kUse; t++) {
+        const uint32_t i = (uint32_t)min(t * kWave + lane, len - 1);
+        c[t] = seg_keys[i];
+        val[t] = seg_values[i];
+    }
+    const uint32_t upper = (uint32_t)bcast_i((int)(uint32_t)(c[0] >> 32), 0);
     bool mixed = false;
 #pragma unroll
     for (int t = 0; t < kUse; t++) {
-        const int i = t * kWave + lane;
-        c[t] = ~0ull;
-        if (i < len) {
-            const uint64_t kk = keys[lo + i];
-            c[t] = (kk << 32) | (uint32_t)i;
-            s_v[i] = values[lo + i];
-            mixed = mixed || (uint32_t)(kk >> 32) != upper;
-        }
+        const bool valid = t * kWave + lane < len;
+        mixed = mixed || (uint32_t)(c[t] >> 32) != upper;
+        c[t] = valid ? c[t] << 32 : ~0ull;
+        val[t] = valid ? val[t] : ~0u;
     }
     if (ballot(mixed)) {     // keys differ above the depth word: left to the general kernel
         if (seg_flags && lane == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
         return;
     }
-    bitonic_network<kUse>(c, lane);
-    __builtin_amdgcn_wave_barrier();
+    bool descends = false;   // position i + 1 holds a smaller value than position i
 #pragma unroll
     for (int t = 0; t < kUse; t++) {
-        const int r = lane * kUse + t;
-        if (r < len) {
-            s_depth[r] = (uint32_t)(c[t] >> 32);
-            s_value[r] = s_v[(uint32_t)c[t]];
+        uint32_t next = (uint32_t)__shfl_down((int)val[t], 1);
+        if (t + 1 < kUse) {
+            const uint32_t wrap = (uint32_t)bcast_i((int)val[t + 1 < kUse ? t + 1 : t], 0);
+            if (lane == kWave - 1) next = wrap;
         }
+        descends = descends || (t * kWave + lane + 1 < len && next < val[t]);
+    }
+    const bool by_value = ballot(descends) == 0;
+    uint32_t* const s_val = (uint32_t*)s_w;
+    if (by_value) {
+#pragma unroll
+        for (int t = 0; t < kUse; t++) c[t] |= val[t];            // the padding stays all ones
+    } else {
+#pragma unroll
+        for (int t = 0; t < kUse; t++) {
+            const int i = t * kWave + lane;
+            if (i < len) { s_val[i] = val[t]; c[t] |= (uint32_t)i; }
+        }
+    }
+    bitonic_network<kUse>(c, lane);
+    asm volatile("" : "+v"(lane));
+    if (!by_value) {
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int t = 0; t < kUse; t++)
+            if (lane * kUse + t < len) c[t] = (c[t] & 0xffffffff00000000ull) | s_val[(uint32_t)c[t]];
     }
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int t = 0; t < kUse; t++) {
+        const int r = lane * kUse + t;
+        if (r < len) s_w[staged(r)] = c[t];
+    }
+    __builtin_amdgcn_wave_barrier();
+    uint64_t* const key_to = keys + lo + lane;
+    uint32_t* const value_to = values + lo + lane;
+#pragma unroll
+    for (int t = 0; t < kUse; t++) {
         const int i = t * kWave + lane;
         if (i < len) {
-            keys[lo + i] = ((uint64_t)upper << 32) | s_depth[i];
-            values[lo + i] = s_value[i];
+            const uint64_t w = s_w[staged(i)];
+            key_to[t * kWave] = ((uint64_t)upper << 32) | (w >> 32);
+            value_to[t * kWave] = (uint32_t)w;
         }
     }
     __builtin_amdgcn_wave_barrier();
 }
 
 // The network over the smallest power of two of register slots (at most kT) that holds the segment.
-// s_v: 3 * kT * 64 words.
+// s_w: staging_words(64 * kT) 64-bit words.
 template <int kT>
 __device__ __forceinline__ void sort_segment_bitonic(uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
                                                      uint32_t v, int lo, int hi, uint32_t* __restrict__ seg_flags,
-                                                     uint32_t* s_v)
+                                                     uint64_t* s_w)
 {
-    constexpr int kS = kT * kWave;
     const int len = hi - lo;
-    if (len <= kWave) sort_segment_bitonic_of<1, kS>(keys, values, v, lo, hi, seg_flags, s_v);
-    else if (kT >= 2 && len <= 2 * kWave) sort_segment_bitonic_of<(kT >= 2 ? 2 : 1), kS>(keys, values, v, lo, hi, seg_flags, s_v);
-    else if (kT >= 4 && len <= 4 * kWave) sort_segment_bitonic_of<(kT >= 4 ? 4 : 1), kS>(keys, values, v, lo, hi, seg_flags, s_v);
-    else if (kT >= 8 && len <= 8 * kWave) sort_segment_bitonic_of<(kT >= 8 ? 8 : 1), kS>(keys, values, v, lo, hi, seg_flags, s_v);
-    else sort_segment_bitonic_of<kT, kS>(keys, values, v, lo, hi, seg_flags, s_v);
+    if (len <= kWave) sort_segment_bitonic_of<1>(keys, values, v, lo, hi, seg_flags, s_w);
+    else if (kT >= 2 && len <= 2 * kWave) sort_segment_bitonic_of<(kT >= 2 ? 2 : 1)>(keys, values, v, lo, hi, seg_flags, s_w);
+    else if (kT >= 4 && len <= 4 * kWave) sort_segment_bitonic_of<(kT >= 4 ? 4 : 1)>(keys, values, v, lo, hi, seg_flags, s_w);
+    else if (kT >= 8 && len <= 8 * kWave) sort_segment_bitonic_of<(kT >= 8 ? 8 : 1)>(keys, values, v, lo, hi, seg_flags, s_w);
+    else sort_segment_bitonic_of<kT>(keys, values, v, lo, hi, seg_flags, s_w);
 }
 
 // One wave per workgroup; with a table of segment starts the workgroup looks at kIds tile ids
@@ -946,38 +1075,41 @@ __global__ __launch_bounds__(kWave) void segment_sort_wave_kernel(
     uint32_t* __restrict__ list2, uint32_t* __restrict__ list3,
     uint32_t list_cap0, uint32_t list_cap1, uint32_t list_cap2, uint32_t list_cap3)
 {
-    __shared__ uint32_t s_v[3 * kT * kWave];      // values by position, sorted depths, sorted values
+    __shared__ uint64_t s_w[staging_words(kT * kWave)];
     const int lane = threadIdx.x;
+    uint32_t first_id = blockIdx.x;
+    uint64_t todo = 0;
+    int lo_found = 0, hi_found = 0;
     if (!seg_start) {
-        const uint32_t v = blockIdx.x;
-        const int lo = wave_lower_bound(keys, n, v, tile_mask);
-        const int hi = v == tile_mask ? n : wave_lower_bound(keys, n, v + 1, tile_mask);
-        if (hi - lo <= min_len || hi - lo > kT * kWave) return;
-        sort_segment_bitonic<kT>(keys, values, v, lo, hi, seg_flags, s_v);
-        return;
+        lo_found = wave_lower_bound(keys, n, first_id, tile_mask);
+        hi_found = first_id == tile_mask ? n : wave_lower_bound(keys, n, first_id + 1, tile_mask);
+        todo = hi_found - lo_found > min_len && hi_found - lo_found <= kT * kWave ? 1u : 0u;
+    } else {
+        first_id = blockIdx.x * (uint32_t)kIds;
+        const uint32_t mine = first_id + (uint32_t)lane;
+        int len = 0;
+        if (lane < kIds && mine < ids) len = seg_start[mine + 1] - seg_start[mine];
+        // This launch sees every tile id once: it also lists the ids of the longer segments by class
+        // (lengths up to list_max0, list_max1, list_max2, and everything longer), so that those
+        // fewer, longer-running segments can be dealt out evenly by the launches that follow.
+        if (list0) {
+            // neighbouring tiles tend to be equally busy: mix the index so that every list gets its share
+            const uint32_t shard = (blockIdx.x ^ (blockIdx.x >> 5) ^ (blockIdx.x >> 10) ^ (blockIdx.x >> 15)) % kListShards;
+            if (len > kT * kWave && len <= list_max0)
+                list0[(size_t)shard * list_cap0 + atomicAdd(&seg_counts[0 * kListShards + shard], 1u)] = mine;
+            else if (len > list_max0 && len <= list_max1)
+                list1[(size_t)shard * list_cap1 + atomicAdd(&seg_counts[1 * kListShards + shard], 1u)] = mine;
+            else if (len > list_max1 && len <= list_max2)
+                list2[(size_t)shard * list_cap2 + atomicAdd(&seg_counts[2 * kListShards + shard], 1u)] = mine;
+            else if (len > list_max2)
+                list3[(size_t)shard * list_cap3 + atomicAdd(&seg_counts[3 * kListShards + shard], 1u)] = mine;
+        }
+        todo = ballot(len > min_len && len <= kT * kWave);
     }
-    const uint32_t first_id = blockIdx.x * (uint32_t)kIds;
-    const uint32_t mine = first_id + (uint32_t)lane;
-    int len = 0;
-    if (lane < kIds && mine < ids) len = seg_start[mine + 1] - seg_start[mine];
-    // This launch sees every tile id once: it also lists the ids of the longer segments by class
-    // (lengths up to list_max0, list_max1, list_max2, and everything longer), so that those
-    // fewer, longer-running segments can be dealt out evenly by the launches that follow.
-    if (list0) {
-        // neighbouring tiles tend to be equally busy: mix the index so that every list gets its share
-        const uint32_t shard = (blockIdx.x ^ (blockIdx.x >> 5) ^ (blockIdx.x >> 10) ^ (blockIdx.x >> 15)) % kListShards;
-        if (len > kT * kWave && len <= list_max0)
-            list0[(size_t)shard * list_cap0 + atomicAdd(&seg_counts[0 * kListShards + shard], 1u)] = mine;
-        else if (len > list_max0 && len <= list_max1)
-            list1[(size_t)shard * list_cap1 + atomicAdd(&seg_counts[1 * kListShards + shard], 1u)] = mine;
-        else if (len > list_max1 && len <= list_max2)
-            list2[(size_t)shard * list_cap2 + atomicAdd(&seg_counts[2 * kListShards + shard], 1u)] = mine;
-        else if (len > list_max2)
-            list3[(size_t)shard * list_cap3 + atomicAdd(&seg_counts[3 * kListShards + shard], 1u)] = mine;
-    }
-    for (uint64_t todo = ballot(len > min_len && len <= kT * kWave); todo; todo &= todo - 1) {
+    for (; todo; todo &= todo - 1) {
         const uint32_t v = first_id + (uint32_t)(__ffsll((long long)todo) - 1);
-        sort_segment_bitonic<kT>(keys, values, v, seg_start[v], seg_start[v + 1], seg_flags, s_v);
+        const int lo = seg_start ? seg_start[v] : lo_found, hi = seg_start ? seg_start[v + 1] : hi_found;
+        sort_segment_bitonic<kT>(keys, values, v, lo, hi, seg_flags, s_w);
         __builtin_amdgcn_wave_barrier();
     }
 }
@@ -990,12 +1122,12 @@ __global__ __launch_bounds__(kWave) void segment_sort_wave_list_kernel(
     uint32_t* __restrict__ seg_flags, const uint32_t* __restrict__ list, const uint32_t* __restrict__ list_count,
     uint32_t list_cap)
 {
-    __shared__ uint32_t s_v[3 * kT * kWave];      // values by position, sorted depths, sorted values
+    __shared__ uint64_t s_w[staging_words(kT * kWave)];
     const uint32_t shard = blockIdx.x % kListShards;
     const uint32_t count = list_count[shard];
     for (uint32_t i = blockIdx.x / kListShards; i < count; i += gridDim.x / kListShards) {
         const uint32_t v = list[(size_t)shard * list_cap + i];
-        sort_segment_bitonic<kT>(keys, values, v, seg_start[v], seg_start[v + 1], seg_flags, s_v);
+        sort_segment_bitonic<kT>(keys, values, v, seg_start[v], seg_start[v + 1], seg_flags, s_w);
         __builtin_amdgcn_wave_barrier();
     }
 }
@@ -1049,9 +1181,9 @@ __global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_ke
     const uint32_t* __restrict__ list_medium, uint32_t cap_medium, const uint32_t* __restrict__ list_large, uint32_t cap_large)
 {
     constexpr int kLdsCap = kAllClasses ? kCapLarge : 1;
-    __shared__ uint32_t s_k[2][kLdsCap];
-    __shared__ uint32_t s_v[2][kLdsCap];
-    __shared__ uint32_t s_cnt[kGeneralWaves][kBins];
+    __shared__ uint32_t s_k[kLdsCap];
+    __shared__ uint32_t s_v[kLdsCap];
+    __shared__ uint32_t s_cnt[kGeneralWaves][kBins];      // the passes in LDS use it as 16-bit counters
     __shared__ uint32_t s_wave_sum[kGeneralWaves];
     __shared__ int s_bounds[2];
     __shared__ int s_flag;
@@ -1098,7 +1230,7 @@ __global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_ke
                     // keys that differ above the depth word: through memory right away (no flag: the
                     // workgroups that look at the flags run beside this one)
                     if (sort_segment_lds<kGeneralWaves, kCapLarge>(keys, values, v, seg_start[v], seg_start[v + 1], nullptr,
-                                                                   s_k, s_v, s_cnt, s_wave_sum, &s_flag))
+                                                                   s_k, s_v, (uint16_t (*)[kBins])s_cnt, s_wave_sum, &s_flag))
                         sort_segment_general(keys, values, alt_keys, alt_values, seg_start[v], seg_start[v + 1], s_cnt, s_wave_sum, &s_flag);
                 }
             }
@@ -1128,8 +1260,6 @@ __global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_ke
     }
 }
 
-constexpr int kMergedTailMax = 1 << 19;      // up to this many pairs the last launch also takes the classes of 1025 .. 8192 pairs
-constexpr uint32_t kOneLaunchIds = 32768;    // up to this many tile ids one launch sorts every segment of up to kCapSmall pairs
 
 
 } // namespace
@@ -1194,6 +1324,8 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         seg_counts = (uint32_t*)(list_sorting_space + ws.seg_lists);
     }
     bool table_by_scatter = false;
+    const bool one_wave_launch = seg_start && ids <= kOneLaunchIds;
+    const uint32_t flag_words = (ids + 31) / 32;
 
     // 1. stable partition by tile id, least significant tile digit first
     auto partition = [&](auto shape) {
@@ -1212,12 +1344,12 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
             const bool last = p == passes - 1;
             if (g.tiles <= kSmallRows) {
                 hipLaunchKernelGGL((count_kernel<Shape>), dim3(g.tiles), dim3(kSortBlock), 0, st, src_k, n, shift, nbits, hist,
-                                   last ? seg_flags : nullptr, (ids + 31) / 32, seg_counts);
+                                   last ? seg_flags : nullptr, flag_words, seg_counts);
             } else {
                 const int groups = g.chunk < kCountGroups ? g.chunk : kCountGroups;
                 hipLaunchKernelGGL((count_chunk_kernel<Shape>), dim3(g.chunks), dim3(groups * kSortBlock), 0, st,
                                    src_k, n, shift, nbits, hist, g.tiles, g.chunk, chunk_sums,
-                                   last ? seg_flags : nullptr, (ids + 31) / 32, seg_counts);
+                                   last ? seg_flags : nullptr, flag_words, seg_counts);
                 hipLaunchKernelGGL((offsets_kernel<Shape>), dim3(g.chunks), dim3(g.chunks > 16 ? kOffsetThreads : Shape::kBinsP), 0, st,
                                    hist, g.tiles, g.chunk, chunk_sums, g.chunks);
             }
@@ -1239,7 +1371,7 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         if (seg_start && !table_by_scatter) {
             const unsigned blocks = (unsigned)(((size_t)n + 256 * kStartsPerThread - 1) / (256 * kStartsPerThread));
             hipLaunchKernelGGL(segment_starts_kernel, dim3(blocks), dim3(256), 0, st,
-                               (const uint64_t*)gaussian_keys_sorted, n, tile_mask, ids, seg_start, seg_flags, seg_counts);
+                               (const uint64_t*)gaussian_keys_sorted, n, tile_mask, ids, seg_start, seg_flags, flag_words, seg_counts);
         }
         uint64_t* ks = gaussian_keys_sorted;
         uint32_t* vs = gaussian_values_sorted;
@@ -1267,7 +1399,6 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         // launch of their own lasts as long as one such sort: there the first launch takes them
         // too, with 16 register slots (1080p: -15 us, 4K: -8 us; at 8K +40 us, because the launch
         // over 131 072 ids, most of them under 128 pairs, then runs at fewer waves per SIMD).
-        const bool one_wave_launch = seg_start && ids <= kOneLaunchIds;
         if (one_wave_launch)
             hipLaunchKernelGGL((segment_sort_wave_kernel<kCapSmall / kWave, 1>), dim3(ids), dim3(kWave),
                                0, st, ks, vs, n, tile_mask, 1, ids, (const int*)seg_start, seg_flags,
