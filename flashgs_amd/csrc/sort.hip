@@ -947,10 +947,10 @@ __device__ __forceinline__ void bitonic_network(uint64_t (&c)[kT], int lane)
     }
 }
 
-// Words of LDS a wave needs to sort up to n pairs with the network: one 64-bit word per pair, one
-// word of padding after every 16 (lane l puts its kUse consecutive ranks down at once; without
+// Words of LDS a wave needs to sort up to n pairs with the network: one 64-bit word for every
+// second pair (the sorted pairs go through it in two halves), one word of padding after every 16 (lane l puts its kUse consecutive ranks down at once; without
 // the padding the lanes of a wave would all start in the same bank).
-__host__ __device__ constexpr int staging_words(int n) { return n + n / 16; }
+__host__ __device__ constexpr int staging_words(int n) { return n <= 64 ? n + n / 16 : n / 2 + n / 32; }
 __device__ __forceinline__ int staged(int i) { return i + (i >> 4); }
 
 // Sorts the segment [lo, hi) of tile id v with the network over kUse slots per lane, 64 * kUse >= hi - lo.
@@ -974,28 +974,26 @@ __device__ __forceinline__ void sort_segment_bitonic_of(uint64_t* __restrict__ k
     const int len = hi - lo;
     uint64_t c[kUse];
     uint32_t val[kUse];
-    const uint64_t* const seg_keys = keys + lo;
-    const uint32_t* const seg_values = values + lo;
-    // Every load is issued before the first one is looked at: a slot past the end of the segment
-    // reads the last pair again (a load under a condition would be waited for before the next).
+    // Every load is issued before the first one is looked at (nothing but the load stands under
+    // the condition: a use in there would be waited for before the next slot's load goes out).  A
+    // slot past the end of the segment keeps all ones and sorts behind every pair.
+    const uint64_t* const key_at = keys + lo + lane;
+    const uint32_t* const value_at = values + lo + lane;
 #pragma unroll
     for (int t = 0; t < kUse; t++) {
-        const uint32_t i = (uint32_t)min(t * kWave + lane, len - 1);
-        c[t] = seg_keys[i];
-        val[t] = seg_values[i];
+        c[t] = ~0ull;
+        val[t] = ~0u;
+        if (t * kWave + lane < len) {
+            c[t] = key_at[t * kWave];
+            val[t] = value_at[t * kWave];
+        }
     }
     const uint32_t upper = (uint32_t)bcast_i((int)(uint32_t)(c[0] >> 32), 0);
     bool mixed = false;
 #pragma unroll
     for (int t = 0; t < kUse; t++) {
-        const bool valid = t * kWave + lane < len;
-        mixed = mixed || (uint32_t)(c[t] >> 32) != upper;
-        c[t] = valid ? c[t] << 32 : ~0ull;
-        val[t] = valid ? val[t] : ~0u;
-    }
-    if (ballot(mixed)) {     // keys differ above the depth word: left to the general kernel
-        if (seg_flags && lane == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
-        return;
+        mixed = mixed || (t * kWave + lane < len && (uint32_t)(c[t] >> 32) != upper);
+        c[t] <<= 32;                                                // the padding: depth of all ones
     }
     bool descends = false;   // position i + 1 holds a smaller value than position i
 #pragma unroll
@@ -1007,42 +1005,54 @@ __device__ __forceinline__ void sort_segment_bitonic_of(uint64_t* __restrict__ k
         }
         descends = descends || (t * kWave + lane + 1 < len && next < val[t]);
     }
+    // (looked at behind the values on purpose: in front of them, their loads would wait for it)
+    if (ballot(mixed)) {     // keys differ above the depth word: left to the general kernel
+        if (seg_flags && lane == 0) atomicOr(&seg_flags[v >> 5], 1u << (v & 31));
+        return;
+    }
     const bool by_value = ballot(descends) == 0;
+    // (no branches around the slots: where two paths meet, the sixteen words are copied from the
+    // registers one path left them in to those of the other)
     uint32_t* const s_val = (uint32_t*)s_w;
-    if (by_value) {
-#pragma unroll
-        for (int t = 0; t < kUse; t++) c[t] |= val[t];            // the padding stays all ones
-    } else {
-#pragma unroll
-        for (int t = 0; t < kUse; t++) {
-            const int i = t * kWave + lane;
-            if (i < len) { s_val[i] = val[t]; c[t] |= (uint32_t)i; }
-        }
-    }
-    bitonic_network<kUse>(c, lane);
-    asm volatile("" : "+v"(lane));
-    if (!by_value) {
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int t = 0; t < kUse; t++)
-            if (lane * kUse + t < len) c[t] = (c[t] & 0xffffffff00000000ull) | s_val[(uint32_t)c[t]];
-    }
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int t = 0; t < kUse; t++) {
-        const int r = lane * kUse + t;
-        if (r < len) s_w[staged(r)] = c[t];
-    }
-    __builtin_amdgcn_wave_barrier();
-    uint64_t* const key_to = keys + lo + lane;
-    uint32_t* const value_to = values + lo + lane;
 #pragma unroll
     for (int t = 0; t < kUse; t++) {
         const int i = t * kWave + lane;
-        if (i < len) {
-            const uint64_t w = s_w[staged(i)];
-            key_to[t * kWave] = ((uint64_t)upper << 32) | (w >> 32);
-            value_to[t * kWave] = (uint32_t)w;
+        if (!by_value && i < len) s_val[i] = val[t];
+        c[t] |= by_value || i >= len ? val[t] : (uint32_t)i;     // the padding stays all ones
+    }
+    bitonic_network<kUse>(c, lane);
+    asm volatile("" : "+v"(lane));
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int t = 0; t < kUse; t++) {
+        const uint32_t low = (uint32_t)c[t];
+        const uint32_t looked_up = s_val[by_value ? 0u : min(low, (uint32_t)(kUse * kWave - 1))];
+        c[t] = (c[t] & 0xffffffff00000000ull) | (by_value ? low : looked_up);
+    }
+    // back to contiguous stores through LDS, the lower half of the ranks (lanes 0..31) first, then
+    // the upper half through the same words: half the LDS, twice the waves per CU
+    constexpr int kRounds = kUse >= 2 ? 2 : 1, kPart = kUse * kWave / kRounds;
+    uint64_t* const key_to = keys + lo + lane;
+    uint32_t* const value_to = values + lo + lane;
+#pragma unroll
+    for (int h = 0; h < kRounds; h++) {
+        __builtin_amdgcn_wave_barrier();
+        if (lane / (kWave / kRounds) == h) {
+#pragma unroll
+            for (int t = 0; t < kUse; t++) {
+                const int r = lane * kUse + t;
+                if (r < len) s_w[staged(r - h * kPart)] = c[t];
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int t = h * (kUse / kRounds); t < (h + 1) * (kUse / kRounds); t++) {
+            const int i = t * kWave + lane;
+            if (i < len) {
+                const uint64_t w = s_w[staged(i - h * kPart)];
+                key_to[t * kWave] = ((uint64_t)upper << 32) | (w >> 32);
+                value_to[t * kWave] = (uint32_t)w;
+            }
         }
     }
     __builtin_amdgcn_wave_barrier();
