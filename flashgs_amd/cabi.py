@@ -22,6 +22,9 @@ SIGNATURES = {
                        + [C.c_void_p] * 6 + [C.c_int64, C.c_void_p]),
     "fgs_preprocess_static": (C.c_int, [C.c_int] + [C.c_void_p] * 4 + [C.c_int] * 4 + [C.c_void_p] * 2 + [C.c_float] * 4
                               + [C.c_void_p] * 6 + [C.c_int64, C.c_void_p]),
+    "fgs_preprocess_mirrored": (C.c_int, [C.c_int] + [C.c_void_p] * 4 + [C.c_int] * 4 + [C.c_void_p] * 2 + [C.c_float] * 4
+                                + [C.c_void_p] * 6 + [C.c_int64, C.c_void_p, C.c_void_p]),
+    "fgs_wait_count": (C.c_int, [C.c_void_p, C.c_double, C.c_void_p]),
     "fgs_sort_gaussian": (C.c_int, [C.c_int] * 5 + [C.c_void_p, C.c_size_t] + [C.c_void_p] * 4 + [C.c_void_p]),
     "fgs_get_sort_buffer_size": (C.c_size_t, [C.c_int]),
     "fgs_render_16x16": (C.c_int, _RENDER_ARGS),
@@ -84,17 +87,31 @@ def camera_matrices(position, rotation, width, height, focal_x, focal_y, zFar, z
     return view, proj
 
 
+COUNT_PENDING = -2147483647       # FGS_COUNT_PENDING: what the caller puts into the count mirror before the call
+
+
 def preprocess(P, positions, shs, opacities, cov3ds, width, height, block_x, block_y, position, rotation,
                focal_x, focal_y, zFar, zNear, points_xy, rgb_depth, conic_opacity, keys, values, curr_offset,
-               key_capacity=0, stream=0, static=False):
-    """``static=True`` calls fgs_preprocess_static, the variant that allocates nothing."""
+               key_capacity=0, stream=0, static=False, count_mirror=None):
+    """``static=True`` calls fgs_preprocess_static, the variant that allocates nothing;
+    ``count_mirror`` (address of a word of pinned host memory holding COUNT_PENDING) calls
+    fgs_preprocess_mirrored, which also stores the pair count there for `wait_count`."""
     pos, rot = _host_f32(position, 3), _host_f32(rotation, 9)
-    fn = load().fgs_preprocess_static if static else load().fgs_preprocess
-    rc = fn(P, positions, shs, opacities, cov3ds, width, height, block_x, block_y,
+    name = "fgs_preprocess_mirrored" if count_mirror is not None else "fgs_preprocess_static" if static else "fgs_preprocess"
+    if count_mirror is not None and static:
+        raise ValueError("static and count_mirror exclude each other")
+    tail = (key_capacity, count_mirror, stream) if count_mirror is not None else (key_capacity, stream)
+    rc = getattr(load(), name)(P, positions, shs, opacities, cov3ds, width, height, block_x, block_y,
                                pos.ctypes.data, rot.ctypes.data, focal_x, focal_y, zFar, zNear,
-                               points_xy, rgb_depth, conic_opacity, keys, values, curr_offset,
-            key_capacity, stream)
-    _check(rc, "fgs_preprocess_static" if static else "fgs_preprocess")
+                               points_xy, rgb_depth, conic_opacity, keys, values, curr_offset, *tail)
+    _check(rc, name)
+
+
+def wait_count(count_mirror, timeout_seconds=10.0):
+    """Polls the count mirror of a `preprocess(..., count_mirror=...)` call; the pair count (negative: the launch gave up)."""
+    out = C.c_int(0)
+    _check(load().fgs_wait_count(count_mirror, float(timeout_seconds), C.addressof(out)), "fgs_wait_count")
+    return out.value
 
 
 COLOUR_SUMS_MATRIX_F16, COLOUR_SUMS_FP32 = 0, 1

@@ -23,6 +23,7 @@
 #include "fgs_internal.h"
 
 #include <atomic>
+#include <chrono>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -375,6 +376,12 @@ __device__ __forceinline__ uint64_t peek(const uint64_t* slot)
     return __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// The pair count (or INT_MIN) for a host that polls for it: `mirror` is pinned host memory.
+__device__ __forceinline__ void report_count(int* mirror, int value)
+{
+    if (mirror) __hip_atomic_store(mirror, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // The scanner: one wave.  Reads the workgroups' counts in order, kScanPerLane consecutive ones
 // per lane and trip, and writes the exclusive running sum of every count that is there and has no
 // gap in front of it; then goes on from the first gap.  What counts is how soon after a count an
@@ -383,7 +390,7 @@ __device__ __forceinline__ uint64_t peek(const uint64_t* slot)
 constexpr int kScanPerLane = 2;
 
 __device__ __forceinline__ bool scan_counts(const uint64_t* counts, uint64_t* offsets, int num_blocks,
-                                            int* curr_offset, unsigned spin_limit)
+                                            int* curr_offset, int* count_mirror, unsigned spin_limit)
 {
     const int lane = lane_id();
     const uint32_t start = (uint32_t)*curr_offset;      // the caller's starting offset (example.py:69 zeroes it)
@@ -425,9 +432,12 @@ __device__ __forceinline__ bool scan_counts(const uint64_t* counts, uint64_t* of
     }
     if (gave_up) {
         for (int j = base + lane; j < num_blocks; j += kWave) publish(offsets + j, pack_status(kStatePoison, 0u));
-        if (lane == 0) atomicMin(curr_offset, kIntMin);
+        if (lane == 0) { atomicMin(curr_offset, kIntMin); report_count(count_mirror, kIntMin); }
     } else if (lane == 0) {
-        atomicCAS(curr_offset, (int)start, (int)running);
+        // the total is known here, while workgroups are still writing their keys: a host that polls
+        // the mirror can launch the sort behind this launch that much earlier
+        const int found = atomicCAS(curr_offset, (int)start, (int)running);
+        report_count(count_mirror, found == (int)start ? (int)running : kIntMin);
     }
     return gave_up;
 }
@@ -464,7 +474,8 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     uint64_t* __restrict__ scan_words,     // control word, then two generations of (counts, offsets), status_capacity words each
     int status_capacity,
     int num_blocks,                        // workgroups that hold Gaussians; the grid has one more, the scanner's
-    unsigned spin_limit)
+    unsigned spin_limit,
+    int* __restrict__ count_mirror)        // pinned host memory that also receives the pair count, or null
 {
     __shared__ uint32_t s_wave_total[kWavesPerBlock];
     __shared__ uint32_t s_block_base;
@@ -494,7 +505,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     const uint32_t control = s_control;
     if (control & kControlAborted) {
         // a scanner on these words gave up (in this launch or an earlier one): touch nothing
-        if (tid == 0) atomicMin(curr_offset, kIntMin);
+        if (tid == 0) { atomicMin(curr_offset, kIntMin); if (blockIdx.x == 0) report_count(count_mirror, kIntMin); }
         return;
     }
 
@@ -512,7 +523,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     // later one waits for its offset (and every wait is bounded in any case).
     if (blockIdx.x == 0) {
         if (wave == 0) {
-            const bool gave_up = scan_counts(counts, offsets, num_blocks, curr_offset, spin_limit);
+            const bool gave_up = scan_counts(counts, offsets, num_blocks, curr_offset, count_mirror, spin_limit);
             // Read every count: every workgroup has read the control word by now, so the other
             // generation can be handed to the next launch.  Gave up: workgroups may still be
             // dispatched; the generation stays and the words are marked unusable.
@@ -875,7 +886,7 @@ __global__ __launch_bounds__(kBlock) void preprocess_kernel(
     if (tid == 0) {
         bool failed = false;
         s_block_base = wait_for_offset(offsets + ticket, spin_limit, &failed);
-        if (failed) atomicMin(curr_offset, kIntMin);
+        if (failed) { atomicMin(curr_offset, kIntMin); report_count(count_mirror, kIntMin); }
     }
     __syncthreads();
     const uint32_t my_slot = s_block_base + wave_base + (incl - count);
@@ -1100,6 +1111,11 @@ int static_scratch(int device, uint64_t** out)
     return FGS_OK;
 }
 
+__global__ void mirror_count_kernel(const int* curr_offset, int* count_mirror)
+{
+    report_count(count_mirror, *curr_offset);
+}
+
 int preprocess_impl(bool allocate, const char* who, int P,
                     const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
                     int width, int height, int block_x, int block_y,
@@ -1107,7 +1123,7 @@ int preprocess_impl(bool allocate, const char* who, int P,
                     float focal_x, float focal_y, float zFar, float zNear,
                     float* points_xy, float* rgb_depth, float* conic_opacity,
                     uint64_t* gaussian_keys_unsorted, uint32_t* gaussian_values_unsorted,
-                    int* curr_offset, int64_t key_capacity, void* stream)
+                    int* curr_offset, int64_t key_capacity, int* count_mirror, void* stream)
 {
     if (P < 0) return fail(FGS_E_INVALID, "%s: P = %d is negative", who, P);
     if (width <= 0 || height <= 0 || block_x <= 0 || block_y <= 0)
@@ -1121,7 +1137,22 @@ int preprocess_impl(bool allocate, const char* who, int P,
     if (!allocate && P > kStaticMaxP)
         return fail(FGS_E_INVALID, "%s: P = %d exceeds the %d Gaussians the built-in scan status holds "
                                    "(fgs_preprocess has no such limit)", who, P, kStaticMaxP);
-    if (P == 0) return FGS_OK;
+    int* mirror_on_device = nullptr;
+    if (count_mirror) {
+        void* mapped = nullptr;
+        if (hipHostGetDevicePointer(&mapped, count_mirror, 0) != hipSuccess || !mapped) {
+            (void)hipGetLastError();
+            return fail(FGS_E_INVALID, "%s: count_mirror must be pinned host memory (hipHostMalloc)", who);
+        }
+        mirror_on_device = (int*)mapped;
+    }
+    if (P == 0) {
+        if (mirror_on_device) {
+            hipLaunchKernelGGL(mirror_count_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, (const int*)curr_offset, mirror_on_device);
+            return check_hip(hipGetLastError(), "mirror_count_kernel launch");
+        }
+        return FGS_OK;
+    }
     if (((uintptr_t)shs | (uintptr_t)rgb_depth | (uintptr_t)conic_opacity) % 16 != 0 ||
         ((uintptr_t)cov3Ds | (uintptr_t)points_xy | (uintptr_t)gaussian_keys_unsorted) % 8 != 0)
         return fail(FGS_E_INVALID, "%s: shs/rgb_depth/conic_opacity must be 16-byte aligned, "
@@ -1167,7 +1198,7 @@ int preprocess_impl(bool allocate, const char* who, int P,
     hipLaunchKernelGGL(preprocess_kernel, dim3(num_blocks + 1), dim3(kBlock), 0, st,
                        P, positions, shs, opacities, cov3Ds, cam, points_xy, rgb_depth, conic_opacity,
                        gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset, key_capacity,
-                       words, status_capacity, num_blocks, g_spin_limit.load());
+                       words, status_capacity, num_blocks, g_spin_limit.load(), mirror_on_device);
     return check_hip(hipGetLastError(), "preprocess_kernel launch");
 }
 
@@ -1211,7 +1242,7 @@ extern "C" int fgs_preprocess(int P,
     return fgs::preprocess_impl(true, "fgs_preprocess", P, positions, shs, opacities, cov3Ds, width, height, block_x, block_y,
                                 cam_position, cam_rotation, focal_x, focal_y, zFar, zNear, points_xy, rgb_depth,
                                 conic_opacity, gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset,
-                                key_capacity, stream);
+                                key_capacity, nullptr, stream);
 }
 
 extern "C" int fgs_preprocess_static(int P,
@@ -1226,5 +1257,39 @@ extern "C" int fgs_preprocess_static(int P,
     return fgs::preprocess_impl(false, "fgs_preprocess_static", P, positions, shs, opacities, cov3Ds, width, height,
                                 block_x, block_y, cam_position, cam_rotation, focal_x, focal_y, zFar, zNear, points_xy,
                                 rgb_depth, conic_opacity, gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset,
-                                key_capacity, stream);
+                                key_capacity, nullptr, stream);
+}
+
+extern "C" int fgs_preprocess_mirrored(int P,
+                                       const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
+                                       int width, int height, int block_x, int block_y,
+                                       const float cam_position[3], const float cam_rotation[9],
+                                       float focal_x, float focal_y, float zFar, float zNear,
+                                       float* points_xy, float* rgb_depth, float* conic_opacity,
+                                       uint64_t* gaussian_keys_unsorted, uint32_t* gaussian_values_unsorted,
+                                       int* curr_offset, int64_t key_capacity, int* count_mirror, void* stream)
+{
+    if (!count_mirror) return fgs::fail(FGS_E_INVALID, "fgs_preprocess_mirrored: null count_mirror");
+    return fgs::preprocess_impl(true, "fgs_preprocess_mirrored", P, positions, shs, opacities, cov3Ds, width, height,
+                                block_x, block_y, cam_position, cam_rotation, focal_x, focal_y, zFar, zNear, points_xy,
+                                rgb_depth, conic_opacity, gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset,
+                                key_capacity, count_mirror, stream);
+}
+
+extern "C" int fgs_wait_count(const int* count_mirror, double timeout_seconds, int* count)
+{
+    if (!count_mirror || !count) return fgs::fail(FGS_E_INVALID, "fgs_wait_count: null argument");
+    const volatile int* const word = count_mirror;
+    const auto start = std::chrono::steady_clock::now();
+    for (unsigned polls = 0;; polls++) {
+        const int seen = *word;
+        if (seen != FGS_COUNT_PENDING) {
+            *count = seen;
+            return FGS_OK;
+        }
+        if ((polls & 1023u) == 1023u &&
+            std::chrono::duration<double>(std::chrono::steady_clock::now() - start).count() > timeout_seconds)
+            return fgs::fail(FGS_E_TIMEOUT, "fgs_wait_count: no pair count within %.3f s", timeout_seconds);
+        __builtin_ia32_pause();
+    }
 }

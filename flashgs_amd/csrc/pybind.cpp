@@ -79,13 +79,13 @@ void* current_stream(const torch::Tensor& on)
 // ---- ops -----------------------------------------------------------------------------------------
 
 // pybind.cpp:122-150
-void preprocess(torch::Tensor& orig_points, torch::Tensor& shs, torch::Tensor& opacities, torch::Tensor& cov3Ds,
-                int width, int height, int block_x, int block_y,
-                torch::Tensor& position, torch::Tensor& rotation,
-                float focal_x, float focal_y, float zFar, float zNear,
-                torch::Tensor& points_xy, torch::Tensor& rgb_depth, torch::Tensor& conic_opacity,
-                torch::Tensor& gaussian_keys_unsorted, torch::Tensor& gaussian_values_unsorted,
-                torch::Tensor& curr_offset)
+void preprocess_to(torch::Tensor& orig_points, torch::Tensor& shs, torch::Tensor& opacities, torch::Tensor& cov3Ds,
+                   int width, int height, int block_x, int block_y,
+                   torch::Tensor& position, torch::Tensor& rotation,
+                   float focal_x, float focal_y, float zFar, float zNear,
+                   torch::Tensor& points_xy, torch::Tensor& rgb_depth, torch::Tensor& conic_opacity,
+                   torch::Tensor& gaussian_keys_unsorted, torch::Tensor& gaussian_values_unsorted,
+                   torch::Tensor& curr_offset, int* count_mirror)
 {
     need(opacities.dim() >= 1, "opacities must have at least one dimension");
     const int64_t P = opacities.size(0);
@@ -106,6 +106,19 @@ void preprocess(torch::Tensor& orig_points, torch::Tensor& shs, torch::Tensor& o
     need(capacity > 0, "gaussian_keys_unsorted / gaussian_values_unsorted are empty");
 
     DeviceScope scope(opacities);
+    if (count_mirror) {
+        *count_mirror = FGS_COUNT_PENDING;
+        fgs_check(fgs_preprocess_mirrored((int)P,
+                                          orig_points.data_ptr<float>(), shs.data_ptr<float>(), opacities.data_ptr<float>(),
+                                          cov3Ds.data_ptr<float>(), width, height, block_x, block_y, pos.data(), rot.data(),
+                                          focal_x, focal_y, zFar, zNear,
+                                          points_xy.data_ptr<float>(), rgb_depth.data_ptr<float>(), conic_opacity.data_ptr<float>(),
+                                          (uint64_t*)gaussian_keys_unsorted.data_ptr<int64_t>(),
+                                          (uint32_t*)gaussian_values_unsorted.data_ptr<int>(),
+                                          curr_offset.data_ptr<int>(), capacity, count_mirror, current_stream(opacities)),
+                  "preprocess_mirrored");
+        return;
+    }
     fgs_check(fgs_preprocess((int)P,
                              orig_points.data_ptr<float>(), shs.data_ptr<float>(), opacities.data_ptr<float>(),
                              cov3Ds.data_ptr<float>(), width, height, block_x, block_y, pos.data(), rot.data(),
@@ -115,6 +128,52 @@ void preprocess(torch::Tensor& orig_points, torch::Tensor& shs, torch::Tensor& o
                              (uint32_t*)gaussian_values_unsorted.data_ptr<int>(),
                              curr_offset.data_ptr<int>(), capacity, current_stream(opacities)),
               "preprocess");
+}
+
+// pybind.cpp:122-150
+void preprocess(torch::Tensor& orig_points, torch::Tensor& shs, torch::Tensor& opacities, torch::Tensor& cov3Ds,
+                int width, int height, int block_x, int block_y,
+                torch::Tensor& position, torch::Tensor& rotation,
+                float focal_x, float focal_y, float zFar, float zNear,
+                torch::Tensor& points_xy, torch::Tensor& rgb_depth, torch::Tensor& conic_opacity,
+                torch::Tensor& gaussian_keys_unsorted, torch::Tensor& gaussian_values_unsorted,
+                torch::Tensor& curr_offset)
+{
+    preprocess_to(orig_points, shs, opacities, cov3Ds, width, height, block_x, block_y, position, rotation,
+                  focal_x, focal_y, zFar, zNear, points_xy, rgb_depth, conic_opacity,
+                  gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset, nullptr);
+}
+
+int* mirror_word(torch::Tensor& count_mirror)
+{
+    need(!count_mirror.is_cuda() && count_mirror.is_pinned() && count_mirror.scalar_type() == torch::kInt32 &&
+             count_mirror.numel() >= 1 && count_mirror.is_contiguous(),
+         "count_mirror must be a pinned int32 host tensor (torch.zeros(1, dtype=torch.int32, pin_memory=True))");
+    return count_mirror.data_ptr<int>();
+}
+
+// No counterpart in the reference: preprocess that also stores the pair count into `count_mirror`,
+// pinned host memory, as soon as the launch knows it (fgs_preprocess_mirrored); wait_count polls it.
+void preprocess_mirrored(torch::Tensor& orig_points, torch::Tensor& shs, torch::Tensor& opacities, torch::Tensor& cov3Ds,
+                         int width, int height, int block_x, int block_y,
+                         torch::Tensor& position, torch::Tensor& rotation,
+                         float focal_x, float focal_y, float zFar, float zNear,
+                         torch::Tensor& points_xy, torch::Tensor& rgb_depth, torch::Tensor& conic_opacity,
+                         torch::Tensor& gaussian_keys_unsorted, torch::Tensor& gaussian_values_unsorted,
+                         torch::Tensor& curr_offset, torch::Tensor& count_mirror)
+{
+    preprocess_to(orig_points, shs, opacities, cov3Ds, width, height, block_x, block_y, position, rotation,
+                  focal_x, focal_y, zFar, zNear, points_xy, rgb_depth, conic_opacity,
+                  gaussian_keys_unsorted, gaussian_values_unsorted, curr_offset, mirror_word(count_mirror));
+}
+
+int wait_count(torch::Tensor& count_mirror, double timeout_seconds)
+{
+    int count = 0;
+    const int* const word = mirror_word(count_mirror);
+    py::gil_scoped_release release;
+    fgs_check(fgs_wait_count(word, timeout_seconds, &count), "wait_count");
+    return count;
 }
 
 // pybind.cpp:152-163
@@ -229,5 +288,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     ops.def("render_16x16", &render<16, 16>, "tile ranges and alpha blending, 16x16 tiles");
     ops.def("render_32x16", &render<32, 16>, "tile ranges and alpha blending, 32x16 tiles");
     ops.def("render_32x32", &render<32, 32>, "tile ranges and alpha blending, 32x32 tiles");
+    ops.def("preprocess_mirrored", &preprocess_mirrored,
+            "preprocess that also stores the pair count into a pinned host tensor as soon as it is known");
+    ops.def("wait_count", &wait_count, "poll the pinned host tensor of preprocess_mirrored for the pair count");
     ops.def("reset_scan", &reset_scan, "clear preprocess's scan status on the tensor's device and current stream");
 }

@@ -1,8 +1,11 @@
 """Driver with the shape of FlashGS's ``example.py``: ``Scene``, ``Camera``, a statically allocated
-``Rasterizer`` whose ``forward`` runs preprocess -> readback -> sort_gaussian -> render_16x16
+``Rasterizer`` whose ``forward`` runs preprocess -> pair count -> sort_gaussian -> render_16x16
 through ``flash_gaussian_splatting.ops``, ``savePpm`` and ``render_scene``.
 
 Differences from the reference driver: the output image is allocated once instead of per frame,
+the pair count is polled in pinned host memory, where the preprocess launch stores it as soon as
+it is known (``ops.preprocess_mirrored`` / ``ops.wait_count``), instead of being copied back with
+a blocking read,
 the too-many-pairs condition raises a real exception (``example.py:82`` raises a string), a
 preprocess whose bounded waits gave up is launched once more after ``ops.reset_scan`` and raises
 ``ScanGaveUp`` if that fails too, and the tile size is a constructor argument.
@@ -109,7 +112,9 @@ class Rasterizer:
         self.points_xy = torch.zeros((scene.num_vertex, 2), device=dev, dtype=torch.float32)
         self.rgb_depth = torch.zeros((scene.num_vertex, 4), device=dev, dtype=torch.float32)
         self.conic_opacity = torch.zeros((scene.num_vertex, 4), device=dev, dtype=torch.float32)
-        self._offset_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        # the launch stores the pair count here as soon as it has it; forward polls this word
+        # instead of the blocking device-to-host copy of example.py:79
+        self._count = torch.zeros(1, dtype=torch.int32, pin_memory=True)
         self._out = None
         if max_width and max_height:
             self._out = torch.zeros((max_height, max_width, 3), device=dev, dtype=torch.uint8)
@@ -126,17 +131,23 @@ class Rasterizer:
         tiles = ((camera.width + bx - 1) // bx) * ((camera.height + by - 1) // by)
         if tiles > self.MAX_NUM_TILES:
             raise ValueError("image needs %d tiles, MAX_NUM_TILES is %d" % (tiles, self.MAX_NUM_TILES))
+        if self.num_rendered >= 0 and int(self._count[0]) < 0:
+            # the count of the last frame was good when it arrived, and a wait of one workgroup gave up after that
+            self.num_rendered = -1
+            o.reset_scan(self.curr_offset)
+            raise ScanGaveUp("a workgroup of the previous frame's preprocess gave up waiting after the pair count "
+                             "had been reported; that frame's image is not to be used")
         for attempt in range(2):
             self.curr_offset.zero_()
-            o.preprocess(scene.position, scene.shs, scene.opacity, scene.cov3d,
-                         camera.width, camera.height, bx, by,
-                         camera.position, camera.rotation,
-                         camera.focal_x, camera.focal_y, camera.zFar, camera.zNear,
-                         self.points_xy, self.rgb_depth, self.conic_opacity,
-                         self.gaussian_keys_unsorted, self.gaussian_values_unsorted, self.curr_offset)
-            # the one blocking device-to-host read of the frame (example.py:79)
-            self._offset_host.copy_(self.curr_offset, non_blocking=False)
-            num_rendered = int(self._offset_host[0])
+            o.preprocess_mirrored(scene.position, scene.shs, scene.opacity, scene.cov3d,
+                                  camera.width, camera.height, bx, by,
+                                  camera.position, camera.rotation,
+                                  camera.focal_x, camera.focal_y, camera.zFar, camera.zNear,
+                                  self.points_xy, self.rgb_depth, self.conic_opacity,
+                                  self.gaussian_keys_unsorted, self.gaussian_values_unsorted, self.curr_offset, self._count)
+            # the count arrives while the launch is still writing keys; the sort below is enqueued
+            # behind it on the same stream
+            num_rendered = o.wait_count(self._count, 60.0)
             if num_rendered >= 0:
                 break
             # a bounded wait of the launch gave up: clear the scan status and launch once more

@@ -24,6 +24,7 @@ extern "C" {
 #define FGS_E_WORKSPACE  -2   /* list_sorting_space too small for num_rendered */
 #define FGS_E_HIP        -3   /* a HIP runtime call or kernel launch failed */
 #define FGS_E_NOMEM      -4   /* internal scratch allocation failed */
+#define FGS_E_TIMEOUT    -5   /* fgs_wait_count: no pair count within the time given */
 
 /* Largest key count the sort accepts (positions and block counts are kept in 32-bit integers). */
 #define FGS_MAX_RENDERED ((1 << 30) - 1)
@@ -92,6 +93,33 @@ int fgs_preprocess_static(int P,
                           float* points_xy, float* rgb_depth, float* conic_opacity,
                           uint64_t* gaussian_keys_unsorted, uint32_t* gaussian_values_unsorted,
                           int* curr_offset, int64_t key_capacity, void* stream);
+
+/*
+ * No counterpart in the reference, whose caller reads the pair count back with a blocking copy
+ * (example.py:79).  fgs_preprocess that also stores the pair count into *count_mirror, a word of
+ * pinned host memory (hipHostMalloc; anything else returns FGS_E_INVALID), for a host that polls
+ * it instead (fgs_wait_count): the caller sets *count_mirror = FGS_COUNT_PENDING before the call.
+ * The count arrives as soon as the launch knows it, which is while it is still writing keys: the
+ * caller can enqueue fgs_sort_gaussian on the same stream at once, stream order does the rest.
+ * A launch that gives up (see fgs_preprocess) stores INT_MIN; if only one workgroup's wait gives up
+ * after the count has been stored, INT_MIN overwrites it later, so a caller that wants to rule
+ * that out looks at the word again, or at *curr_offset, when the stream has drained.
+ */
+#define FGS_COUNT_PENDING (-2147483647)
+int fgs_preprocess_mirrored(int P,
+                            const float* positions, const float* shs, const float* opacities, const float* cov3Ds,
+                            int width, int height, int block_x, int block_y,
+                            const float cam_position[3], const float cam_rotation[9],
+                            float focal_x, float focal_y, float zFar, float zNear,
+                            float* points_xy, float* rgb_depth, float* conic_opacity,
+                            uint64_t* gaussian_keys_unsorted, uint32_t* gaussian_values_unsorted,
+                            int* curr_offset, int64_t key_capacity, int* count_mirror, void* stream);
+
+/*
+ * Host only: polls *count_mirror until it differs from FGS_COUNT_PENDING and stores what it finds
+ * in *count (negative: the launch gave up).  FGS_E_TIMEOUT after timeout_seconds without a count.
+ */
+int fgs_wait_count(const int* count_mirror, double timeout_seconds, int* count);
 
 /*
  * Replaces flashgs::sort_gaussian (csrc/ops.h:41-45, csrc/cuda_rasterizer/sort.cu:28-44):
@@ -243,7 +271,7 @@ const char* fgs_last_error(void);
  * ABI version of this header as major * 1000 + minor: the major number changes when an existing
  * signature or default changes, the minor one when entry points are added.
  */
-#define FGS_ABI_VERSION 2000
+#define FGS_ABI_VERSION 2001
 int fgs_abi_version(void);
 
 #ifdef __cplusplus

@@ -24,9 +24,11 @@ class SceneOnDevice:
         self.cov3d = dev(scene.cov3d)
 
 
-def preprocess(sd, cam, capacity, block=(16, 16), sentinel=None, start_offset=0, guard=True, pad=0, static=False):
+def preprocess(sd, cam, capacity, block=(16, 16), sentinel=None, start_offset=0, guard=True, pad=0, static=False,
+               mirror=False):
     """Returns dict of torch tensors + num_rendered (after a sync).  The key and value buffers are
-    allocated with `pad` entries beyond the capacity the library is told about."""
+    allocated with `pad` entries beyond the capacity the library is told about.  With `mirror` the
+    call is fgs_preprocess_mirrored and `mirrored` is what fgs_wait_count found in the pinned word."""
     n = sd.n
     fillv = 0.0 if sentinel is None else sentinel
     points_xy = torch.full((n, 2), fillv, device=DEV, dtype=torch.float32)
@@ -35,15 +37,18 @@ def preprocess(sd, cam, capacity, block=(16, 16), sentinel=None, start_offset=0,
     keys = torch.zeros(capacity + pad, device=DEV, dtype=torch.int64)
     values = torch.zeros(capacity + pad, device=DEV, dtype=torch.int32)
     curr_offset = torch.full((1,), start_offset, device=DEV, dtype=torch.int32)
+    word = torch.full((1,), cabi.COUNT_PENDING, dtype=torch.int32).pin_memory() if mirror else None
     cabi.preprocess(n, sd.position.data_ptr(), sd.shs.data_ptr(), sd.opacity.data_ptr(), sd.cov3d.data_ptr(),
                     cam.width, cam.height, block[0], block[1], cam.position, cam.rotation,
                     cam.focal_x, cam.focal_y, cam.zFar, cam.zNear,
                     points_xy.data_ptr(), rgb_depth.data_ptr(), conic_opacity.data_ptr(),
                     keys.data_ptr(), values.data_ptr(), curr_offset.data_ptr(),
-                    capacity if guard else 0, torch.cuda.current_stream().cuda_stream, static=static)
+                    capacity if guard else 0, torch.cuda.current_stream().cuda_stream, static=static,
+                    count_mirror=word.data_ptr() if mirror else None)
+    mirrored = cabi.wait_count(word.data_ptr()) if mirror else None
     num = int(curr_offset.cpu()[0])
     return dict(points_xy=points_xy, rgb_depth=rgb_depth, conic_opacity=conic_opacity, keys=keys, values=values,
-                num_rendered=num)
+                num_rendered=num, mirrored=mirrored)
 
 
 def sort(num, width, height, keys, values, block=(16, 16), space_for=None):

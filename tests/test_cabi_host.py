@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), "libflashgs_hip.so does not export %s" % name
         assert name in cabi.SIGNATURES, "flashgs_amd/cabi.py has no binding for %s" % name
-    assert cabi.load().fgs_abi_version() == 2000       # FGS_ABI_VERSION of the header: major * 1000 + minor
+    assert cabi.load().fgs_abi_version() == 2001       # FGS_ABI_VERSION of the header: major * 1000 + minor
 
 
 def test_sort_buffer_size_is_monotonic_and_bounded():
@@ -96,3 +96,24 @@ def test_per_call_blend_flags_are_checked_on_the_host():
         _raises("(-1)", cabi.blend, 16, 16, 64, 64, 256, 256, 256, 256, 256, [0, 0, 0], 256, 0, 0, flags)
         _raises("(-1)", cabi.render_f32, 16, 16, 0, 64, 64, 0, 0, 0, 0, 0, 256, [0, 0, 0], 256, 0, 0, flags)
         assert cabi.blend_kernel_name(16, 16, 64, 64, flags) == ""
+
+
+def test_wait_count_polls_a_host_word():
+    """fgs_wait_count is host code: it returns what it finds in the word once that is not the
+    pending mark (negative counts too), also when it arrives from elsewhere while it polls, and
+    gives up with an error of its own after the time given."""
+    import ctypes as C
+    import threading
+    word = C.c_int(12345)
+    assert cabi.wait_count(C.addressof(word)) == 12345
+    word.value = -2147483648
+    assert cabi.wait_count(C.addressof(word)) == -2147483648
+    word.value = cabi.COUNT_PENDING
+    with pytest.raises(RuntimeError, match="no pair count within"):
+        cabi.wait_count(C.addressof(word), 0.02)
+    timer = threading.Timer(0.05, lambda: setattr(word, "value", 77))
+    timer.start()
+    assert cabi.wait_count(C.addressof(word), 5.0) == 77
+    timer.join()
+    with pytest.raises(RuntimeError, match="null"):
+        cabi.wait_count(None)

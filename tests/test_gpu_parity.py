@@ -274,6 +274,54 @@ def test_start_offset_and_capacity_guard(oracle):
     assert np.all(gp.u64(keys)[cap:] == 0) and np.all(values.cpu().numpy()[cap:] == -1)   # nothing past the capacity
 
 
+def test_mirrored_preprocess_stores_the_count_in_pinned_memory():
+    """fgs_preprocess_mirrored: the word of pinned host memory receives the pair count the launch
+    leaves in *curr_offset (with a starting offset too), everything else is what fgs_preprocess
+    writes; a launch that gives up stores a negative count there; memory that is not pinned is refused."""
+    import gpu_pipeline as gp
+    import torch
+    from flashgs_amd import cabi
+    sc = scenes.config1(n=400_000)
+    cam = sc.cameras[0]
+    sd = gp.SceneOnDevice(sc)
+    cap = 1 << 21
+    plain = gp.preprocess(sd, cam, cap)
+    K = plain["num_rendered"]
+    assert K > 100_000
+    for start in (0, 1000):
+        got = gp.preprocess(sd, cam, cap, start_offset=start, mirror=True)
+        assert got["mirrored"] == got["num_rendered"] == K + start
+        assert np.array_equal(gp.u64(got["keys"])[start:start + K], gp.u64(plain["keys"])[:K])
+        assert np.array_equal(gp.u32(got["values"])[start:start + K], gp.u32(plain["values"])[:K])
+        assert torch.equal(got["rgb_depth"], plain["rgb_depth"])
+    # no Gaussians: the count is the starting offset
+    st = torch.cuda.current_stream().cuda_stream
+    word = torch.full((1,), cabi.COUNT_PENDING, dtype=torch.int32).pin_memory()
+    offset = torch.full((1,), 37, device=gp.DEV, dtype=torch.int32)
+    cabi.preprocess(0, 0, 0, 0, 0, cam.width, cam.height, 16, 16, cam.position, cam.rotation, cam.focal_x, cam.focal_y,
+                    cam.zFar, cam.zNear, 0, 0, 0, 0, 0, offset.data_ptr(), 0, st, count_mirror=word.data_ptr())
+    assert cabi.wait_count(word.data_ptr()) == 37
+    # a launch whose scan gives up
+    previous = cabi.set_scan_spin_limit(0)
+    try:
+        bad = gp.preprocess(gp.SceneOnDevice(scenes.config0(n=1_200_000)), scenes.config0(n=1_200_000).cameras[0], 1 << 22,
+                            mirror=True)
+    finally:
+        cabi.set_scan_spin_limit(previous)
+    assert bad["num_rendered"] < 0 and bad["mirrored"] < 0
+    cabi.reset_scan(st)
+    again = gp.preprocess(sd, cam, cap, mirror=True)
+    assert again["mirrored"] == K
+    # pageable memory cannot be written by the launch
+    pageable = torch.full((1,), cabi.COUNT_PENDING, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="pinned"):
+        cabi.preprocess(0, 0, 0, 0, 0, cam.width, cam.height, 16, 16, cam.position, cam.rotation, cam.focal_x, cam.focal_y,
+                        cam.zFar, cam.zNear, 0, 0, 0, 0, 0, offset.data_ptr(), 0, st, count_mirror=pageable.data_ptr())
+    torch.cuda.synchronize()
+    assert int(torch.zeros(1, device=gp.DEV).sum()) == 0          # the refused call left no error behind
+
+
+@pytest.mark.gpu
 def test_scan_that_gives_up_reports_a_negative_count_until_reset():
     """With the spin limit at 0 every wait of the preprocess launch that is not satisfied at its
     first poll gives up: the kernel still runs to its end (no wave is left waiting) and the pair
@@ -826,7 +874,10 @@ def test_config3_more_than_100M_pairs(oracle, config3_scene):
     assert not gp.u64(got["keys"])[cap:].any() and not gp.u32(got["values"])[cap:].any()
 
 
-def _sort_case(tile, depth_bits, W, H, junk=None, seed=0):
+def _sort_case(tile, depth_bits, W, H, junk=None, seed=0, ascending=False):
+    """`ascending`: the values are the input positions, as the pairs of a tile leave the preprocess
+    (ascending Gaussian indices): the sorting networks then break ties of depth by the value itself.
+    Otherwise a random permutation, where they have to carry positions."""
     import gpu_pipeline as gp
     rng = np.random.default_rng(seed)
     n = tile.size
@@ -836,6 +887,10 @@ def _sort_case(tile, depth_bits, W, H, junk=None, seed=0):
     if junk is not None:
         keys = keys | (junk.astype(np.uint64) << np.uint64(end_bit))
     vals = rng.permutation(n).astype(np.uint32)
+    if ascending:
+        vals = np.arange(n, dtype=np.uint32)
+        far = rng.integers(0, n, 3)                      # three tiles' segments that do not ascend among all that do
+        vals[far] = vals[far][::-1] + np.uint32(1 << 30)
     ks, vs = gp.sort(n, W, H, gp.dev(keys.view(np.int64)), gp.dev(vals.view(np.int32)))
     masked = keys & np.uint64((1 << end_bit) - 1)
     order = np.argsort(masked, kind="stable")
@@ -862,8 +917,9 @@ def test_sort_segment_size_classes(seg, dense):
     _sort_case(tile, depth.view(np.uint32), W, H, seed=seg)
 
 
+@pytest.mark.parametrize("ascending", [False, True])
 @pytest.mark.parametrize("W,H", [(1920, 1080), (3840, 2160)])
-def test_sort_every_segment_length_up_to_1100(W, H):
+def test_sort_every_segment_length_up_to_1100(W, H, ascending):
     """One tile per length 1 ... 1100: every padding of the register sorting networks (64, 128, ... 1024
     elements) and the first lengths of the next class, with many equal depths (ties must keep input
     order) and with depths of all magnitudes, 0 and 0xffffffff included.  At 1080p one launch sorts
@@ -877,7 +933,7 @@ def test_sort_every_segment_length_up_to_1100(W, H):
     depth[rng.integers(0, tile.size, 2000)] = 0
     depth[rng.integers(0, tile.size, 2000)] = 0xFFFFFFFF
     order = rng.permutation(tile.size)
-    _sort_case(tile[order], depth[order], W, H, seed=7)
+    _sort_case(tile[order], depth[order], W, H, seed=7, ascending=ascending)
 
 
 def test_sort_bits_above_the_range_stay_with_their_pair():

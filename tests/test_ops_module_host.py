@@ -17,7 +17,7 @@ def ops():
 
 def test_operator_names(ops):
     for name in ("loadPly", "preprocess", "sort_gaussian", "get_sort_buffer_size", "render_16x16", "render_32x16", "render_32x32",
-                 "reset_scan"):
+                 "reset_scan", "preprocess_mirrored", "wait_count"):
         assert callable(getattr(ops, name))
     assert ops.get_sort_buffer_size(2 ** 20) >= 12 * 2 ** 20
     with pytest.raises(RuntimeError):
