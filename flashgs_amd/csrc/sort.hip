@@ -53,11 +53,15 @@ struct PassShape {
 using Narrow = PassShape<8, 16>;
 using Wide = PassShape<9, 15>;
 constexpr int kNarrowMaxTileBits = 16;
+// A short list (the 0.2M pairs of a 720p frame are 49 blocks of 4096) leaves most CUs without a
+// block and every block ranking 16 rounds: there four pairs per thread, four times the blocks.
+using Short = PassShape<8, 4>;
 
 
 // A list of at most kSmallRows blocks needs no launch that turns the histogram rows into starts:
 // the scatter workgroups add the rows up themselves.
 constexpr int kSmallRows = 64;
+constexpr int kShortPairs = kSmallRows * Narrow::kTile;     // up to this many pairs: blocks of Short::kTile, still without that launch
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -94,8 +98,10 @@ Workspace workspace_for(int n)
 {
     Workspace w;
     const PassGrid a = pass_grid(n, Narrow::kTile), b = pass_grid(n, Wide::kTile);
-    const size_t hist = (size_t)a.tiles * Narrow::kBinsP > (size_t)b.tiles * Wide::kBinsP ? (size_t)a.tiles * Narrow::kBinsP
-                                                                                           : (size_t)b.tiles * Wide::kBinsP;
+    size_t hist = (size_t)a.tiles * Narrow::kBinsP > (size_t)b.tiles * Wide::kBinsP ? (size_t)a.tiles * Narrow::kBinsP
+                                                                                     : (size_t)b.tiles * Wide::kBinsP;
+    if (n <= kShortPairs && (size_t)pass_grid(n, Short::kTile).tiles * Short::kBinsP > hist)
+        hist = (size_t)pass_grid(n, Short::kTile).tiles * Short::kBinsP;
     const size_t sums = (size_t)a.chunks * Narrow::kBinsP > (size_t)b.chunks * Wide::kBinsP ? (size_t)a.chunks * Narrow::kBinsP
                                                                                              : (size_t)b.chunks * Wide::kBinsP;
     w.alt_keys = 0;
@@ -1341,6 +1347,7 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
     auto partition = [&](auto shape) {
         using Shape = decltype(shape);
         const PassGrid g = pass_grid(n, Shape::kTile);
+        const bool small = n <= kShortPairs;         // the scatter workgroups add up the histogram rows themselves
         const int passes = (tile_bits + Shape::kBits - 1) / Shape::kBits;
         table_by_scatter = seg_start && passes <= 2;
         const uint64_t* src_k = gaussian_keys_unsorted;
@@ -1352,7 +1359,7 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
             const int shift = 32 + Shape::kBits * p;
             const int nbits = tile_bits - Shape::kBits * p < Shape::kBits ? tile_bits - Shape::kBits * p : Shape::kBits;
             const bool last = p == passes - 1;
-            if (g.tiles <= kSmallRows) {
+            if (small) {
                 hipLaunchKernelGGL((count_kernel<Shape>), dim3(g.tiles), dim3(kSortBlock), 0, st, src_k, n, shift, nbits, hist,
                                    last ? seg_flags : nullptr, flag_words, seg_counts);
             } else {
@@ -1365,16 +1372,20 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
             }
             if (last && table_by_scatter)
                 hipLaunchKernelGGL((scatter_kernel<Shape, true>), dim3(g.tiles), dim3(kSortBlock), 0, st,
-                                   src_k, src_v, dst_k, dst_v, n, shift, nbits, hist, g.tiles <= kSmallRows ? g.tiles : 0, seg_start);
+                                   src_k, src_v, dst_k, dst_v, n, shift, nbits, hist, small ? g.tiles : 0, seg_start);
             else
                 hipLaunchKernelGGL((scatter_kernel<Shape, false>), dim3(g.tiles), dim3(kSortBlock), 0, st,
-                                   src_k, src_v, dst_k, dst_v, n, shift, nbits, hist, g.tiles <= kSmallRows ? g.tiles : 0, (int*)nullptr);
+                                   src_k, src_v, dst_k, dst_v, n, shift, nbits, hist, small ? g.tiles : 0, (int*)nullptr);
             src_k = dst_k;
             src_v = dst_v;
         }
     };
-    if (tile_bits <= kNarrowMaxTileBits) partition(Narrow());
-    else partition(Wide());
+    if (tile_bits <= kNarrowMaxTileBits) {
+        if (n <= kShortPairs) partition(Short());
+        else partition(Narrow());
+    } else {
+        partition(Wide());
+    }
 
     // 2. every tile id's segment by depth, in place in the sorted buffers
     if (n > 1) {
