@@ -518,6 +518,7 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
 
 // size classes of the segments: pairs per segment
 constexpr int kCapTiny = 512, kCapSmall = 1024, kCapMedium = 4096, kCapLarge = 8192;
+constexpr int kMergedLargeMax = 1 << 24;     // up to this many pairs the last launch also takes the class of 4097 .. 8192 pairs
 constexpr int kMergedTailMax = 1 << 19;      // up to this many pairs the last launch also takes the classes of 1025 .. 8192 pairs
 constexpr uint32_t kOneLaunchIds = 32768;    // up to this many tile ids one launch sorts every segment of up to kCapSmall pairs
 
@@ -1184,9 +1185,10 @@ __device__ __forceinline__ void sort_segment_general(uint64_t* __restrict__ keys
 // one segment at a time, round-robin), the workgroups behind them look at 64 tile ids each for
 // shorter segments that were flagged.
 // With kAllClasses the listed blocks first sort the listed segments of the two classes below
-// (1025 .. kCapLarge pairs, in LDS like segment_sort_kernel<16, kCapLarge>), shard by shard like
-// the launches of those classes: a frame with a short list of pairs has few such segments or
-// none, and one launch instead of three is what counts there.
+// (first_class 1: 1025 .. kCapLarge pairs, 2: only those above kCapMedium; in LDS like
+// segment_sort_kernel<16, kCapLarge>), shard by shard like the launches of those classes: a frame
+// with a short list of pairs has few such segments or none, and one launch instead of three is
+// what counts there; up to kMergedLargeMax pairs the class above kCapMedium still has few.
 template <bool kAllClasses>
 __global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_kernel(
     uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
@@ -1194,7 +1196,8 @@ __global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_ke
     int n, uint32_t tile_mask, int min_len, uint32_t ids,
     const int* __restrict__ seg_start, const uint32_t* __restrict__ seg_flags,
     const uint32_t* __restrict__ list, const uint32_t* __restrict__ list_count, uint32_t list_cap, uint32_t list_blocks,
-    const uint32_t* __restrict__ list_medium, uint32_t cap_medium, const uint32_t* __restrict__ list_large, uint32_t cap_large)
+    const uint32_t* __restrict__ list_medium, uint32_t cap_medium, const uint32_t* __restrict__ list_large, uint32_t cap_large,
+    int first_class)
 {
     constexpr int kLdsCap = kAllClasses ? kCapLarge : 1;
     __shared__ uint32_t s_k[kLdsCap];
@@ -1237,7 +1240,7 @@ __global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_ke
         const uint32_t shard = blockIdx.x % kListShards;
         if constexpr (kAllClasses) {
             // list_count: the counters of all classes, class c at c * kListShards (1: medium, 2: large, 3: long)
-            for (int c = 1; c <= 2; c++) {
+            for (int c = first_class; c <= 2; c++) {
                 const uint32_t* const ids_of = c == 1 ? list_medium : list_large;
                 const uint32_t cap = c == 1 ? cap_medium : cap_large;
                 const uint32_t count = list_count[c * kListShards + shard];
@@ -1433,6 +1436,7 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         // A short list of pairs has few segments of more than 1024 pairs, or none: there the one
         // launch below takes those classes too (720p, 0.2M pairs: two launches less).
         const bool merged_tail = seg_start && n <= kMergedTailMax;
+        const bool merged_large = seg_start && !merged_tail && n <= kMergedLargeMax;
         if (seg_start) {
             if (n > kCapTiny && !one_wave_launch)       // 513..1024: the same network over 16 register slots, from the lists
                 hipLaunchKernelGGL((segment_sort_wave_list_kernel<kCapSmall / kWave>),
@@ -1442,7 +1446,7 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
             if (n > kCapSmall && !merged_tail) {
                 FGS_SEGMENT_CLASS(8, kCapMedium, 64, kCapSmall, list_grid((unsigned)(n / (kCapSmall + 1) + 1), 1024u),
                                   list_medium, seg_counts + kListShards, cap_medium);
-                if (n > kCapMedium)
+                if (n > kCapMedium && !merged_large)
                     FGS_SEGMENT_CLASS(16, kCapLarge, 64, kCapMedium, list_grid((unsigned)(n / (kCapMedium + 1) + 1), 256u),
                                       list_large, seg_counts + 2 * kListShards, cap_large);
             }
@@ -1453,20 +1457,22 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         }
 #undef FGS_SEGMENT_CLASS
         // longer segments from their list, one workgroup per segment; behind them the shorter ones that were flagged
-        if (merged_tail) {
-            const unsigned blocks = n > kCapSmall ? list_grid((unsigned)(n / (kCapSmall + 1) + 1), 256u) : 0u;
+        if (merged_tail || merged_large) {
+            const int smallest = merged_tail ? kCapSmall : kCapMedium;
+            const unsigned blocks = n > smallest ? list_grid((unsigned)(n / (smallest + 1) + 1), 256u) : 0u;
             hipLaunchKernelGGL(segment_sort_general_kernel<true>, dim3(blocks + (ids + kWave - 1) / kWave),
                                dim3(kGeneralWaves * kWave), 0, st, ks, vs, alt_keys, alt_values, n, tile_mask, kCapLarge, ids,
                                (const int*)seg_start, (const uint32_t*)seg_flags,
                                (const uint32_t*)list_long, (const uint32_t*)seg_counts, cap_long, blocks,
-                               (const uint32_t*)list_medium, cap_medium, (const uint32_t*)list_large, cap_large);
+                               (const uint32_t*)list_medium, cap_medium, (const uint32_t*)list_large, cap_large,
+                               merged_tail ? 1 : 2);
         } else {
             const unsigned long_blocks = seg_start && n > kCapLarge ? list_grid((unsigned)(n / (kCapLarge + 1) + 1), 2048u) : 0u;
             hipLaunchKernelGGL(segment_sort_general_kernel<false>, dim3(seg_start ? long_blocks + (ids + kWave - 1) / kWave : ids),
                                dim3(kGeneralWaves * kWave), 0, st, ks, vs, alt_keys, alt_values, n, tile_mask, kCapLarge, ids,
                                (const int*)seg_start, (const uint32_t*)seg_flags,
                                (const uint32_t*)list_long, (const uint32_t*)(seg_counts + 3 * kListShards), cap_long, long_blocks,
-                               no_list, 0u, no_list, 0u);
+                               no_list, 0u, no_list, 0u, 0);
         }
     }
     return check_hip(hipGetLastError(), "sort launch");
