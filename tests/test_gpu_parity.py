@@ -321,7 +321,6 @@ def test_mirrored_preprocess_stores_the_count_in_pinned_memory():
     assert int(torch.zeros(1, device=gp.DEV).sum()) == 0          # the refused call left no error behind
 
 
-@pytest.mark.gpu
 def test_scan_that_gives_up_reports_a_negative_count_until_reset():
     """With the spin limit at 0 every wait of the preprocess launch that is not satisfied at its
     first poll gives up: the kernel still runs to its end (no wave is left waiting) and the pair
@@ -387,6 +386,14 @@ def test_rasterizer_relaunches_once_after_a_scan_that_gave_up():
     finally:
         cabi.set_scan_spin_limit(previous)
     # the status is still marked; forward recovers by itself
+    got = rast.forward(scene, cam, bg)
+    assert rast.num_rendered == K and torch.equal(got, want)
+    # a workgroup that gives up after the count has gone out lowers the mirrored count later: the
+    # next forward reports the frame before, once, and renders again after that
+    torch.cuda.synchronize()
+    rast._count[0] = -2147483648
+    with pytest.raises(ScanGaveUp, match="previous frame"):
+        rast.forward(scene, cam, bg)
     got = rast.forward(scene, cam, bg)
     assert rast.num_rendered == K and torch.equal(got, want)
 
@@ -934,6 +941,28 @@ def test_sort_every_segment_length_up_to_1100(W, H, ascending):
     depth[rng.integers(0, tile.size, 2000)] = 0xFFFFFFFF
     order = rng.permutation(tile.size)
     _sort_case(tile[order], depth[order], W, H, seed=7, ascending=ascending)
+
+
+@pytest.mark.parametrize("n,W,H", [(262_144, 1280, 720), (262_145, 1280, 720), (524_288, 1920, 1080), (524_289, 1920, 1080),
+                                   (262_144, 7680, 4320), ((1 << 24) - 1, 3840, 2160), ((1 << 24) + 1, 3840, 2160)])
+def test_sort_around_the_list_lengths_where_the_launches_change(n, W, H):
+    """The partition blocks are smaller up to 262 144 pairs, the last segment launch takes the
+    classes above 1024 pairs up to 2^19 pairs and the one above 4096 up to 2^24: lists of just those
+    lengths and one more, with crowded tiles of every class among evenly filled ones, values in
+    input order (the networks' tie-break) and many equal depths."""
+    rng = np.random.default_rng(n % 1000 + W)
+    tiles = ((W + 15) // 16) * ((H + 15) // 16)
+    tile = rng.integers(0, tiles, n).astype(np.uint32)
+    pos = 0
+    for length in (600, 1024, 1025, 3000, 4096, 4097, 8192, 8193, 20000, 70000):
+        if pos + length > n // 2:
+            break
+        tile[pos:pos + length] = rng.integers(0, tiles)
+        pos += length
+    rng.shuffle(tile)
+    depth = rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32)
+    depth[::7] = depth[3]
+    _sort_case(tile, depth, W, H, seed=n % 97, ascending=True)
 
 
 def test_sort_bits_above_the_range_stay_with_their_pair():
