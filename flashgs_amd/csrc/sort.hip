@@ -1184,12 +1184,17 @@ __device__ __forceinline__ void sort_segment_general(uint64_t* __restrict__ keys
 // ones longer than min_len: neighbouring tiles tend to be equally crowded, so they are dealt out
 // one segment at a time, round-robin), the workgroups behind them look at 64 tile ids each for
 // shorter segments that were flagged.
-// With kAllClasses the listed blocks first sort the listed segments of the two classes below
-// (first_class 1: 1025 .. kCapLarge pairs, 2: only those above kCapMedium; in LDS like
-// segment_sort_kernel<16, kCapLarge>), shard by shard like the launches of those classes: a frame
-// with a short list of pairs has few such segments or none, and one launch instead of three is
-// what counts there; up to kMergedLargeMax pairs the class above kCapMedium still has few.
-template <bool kAllClasses>
+// With a table (kLds) a listed segment of up to kCapHuge pairs is sorted in LDS like the classes
+// below it, sixteen pairs per thread in registers during a pass (a workgroup then has the LDS of
+// its CU to itself): the passes through memory take 7 us each for 12 000 pairs, those in LDS 2.
+// The listed blocks first sort the listed segments of the classes below (first_class 1:
+// 1025 .. kCapLarge pairs, 2: only those above kCapMedium, 3: none; shard by shard like the
+// launches of those classes): a frame with a short list of pairs has few such segments or none,
+// and one launch instead of three is what counts there; up to kMergedLargeMax pairs the class
+// above kCapMedium still has few.
+constexpr int kCapHuge = 16384;
+
+template <bool kLds>
 __global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_kernel(
     uint64_t* __restrict__ keys, uint32_t* __restrict__ values,
     uint64_t* __restrict__ alt_keys, uint32_t* __restrict__ alt_values,
@@ -1199,7 +1204,7 @@ __global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_ke
     const uint32_t* __restrict__ list_medium, uint32_t cap_medium, const uint32_t* __restrict__ list_large, uint32_t cap_large,
     int first_class)
 {
-    constexpr int kLdsCap = kAllClasses ? kCapLarge : 1;
+    constexpr int kLdsCap = kLds ? kCapHuge : 1;
     __shared__ uint32_t s_k[kLdsCap];
     __shared__ uint32_t s_v[kLdsCap];
     __shared__ uint32_t s_cnt[kGeneralWaves][kBins];      // the passes in LDS use it as 16-bit counters
@@ -1238,26 +1243,24 @@ __global__ __launch_bounds__(kGeneralWaves * kWave) void segment_sort_general_ke
 
     if (blockIdx.x < list_blocks) {
         const uint32_t shard = blockIdx.x % kListShards;
-        if constexpr (kAllClasses) {
-            // list_count: the counters of all classes, class c at c * kListShards (1: medium, 2: large, 3: long)
-            for (int c = first_class; c <= 2; c++) {
-                const uint32_t* const ids_of = c == 1 ? list_medium : list_large;
-                const uint32_t cap = c == 1 ? cap_medium : cap_large;
-                const uint32_t count = list_count[c * kListShards + shard];
-                for (uint32_t i = blockIdx.x / kListShards; i < count; i += list_blocks / kListShards) {
-                    const uint32_t v = ids_of[(size_t)shard * cap + i];
+        // list_count: the counters of all classes, class c at c * kListShards (1: medium, 2: large, 3: long)
+        for (int c = first_class; c <= 3; c++) {
+            const uint32_t* const ids_of = c == 1 ? list_medium : c == 2 ? list_large : list;
+            const uint32_t cap = c == 1 ? cap_medium : c == 2 ? cap_large : list_cap;
+            const uint32_t count = list_count[c * kListShards + shard];
+            for (uint32_t i = blockIdx.x / kListShards; i < count; i += list_blocks / kListShards) {
+                const uint32_t v = ids_of[(size_t)shard * cap + i];
+                const int lo = seg_start[v], hi = seg_start[v + 1];
+                bool through_memory = true;
+                if constexpr (kLds) {
                     // keys that differ above the depth word: through memory right away (no flag: the
                     // workgroups that look at the flags run beside this one)
-                    if (sort_segment_lds<kGeneralWaves, kCapLarge>(keys, values, v, seg_start[v], seg_start[v + 1], nullptr,
-                                                                   s_k, s_v, (uint16_t (*)[kBins])s_cnt, s_wave_sum, &s_flag))
-                        sort_segment_general(keys, values, alt_keys, alt_values, seg_start[v], seg_start[v + 1], s_cnt, s_wave_sum, &s_flag);
+                    if (hi - lo <= kCapHuge)
+                        through_memory = sort_segment_lds<kGeneralWaves, kCapHuge>(keys, values, v, lo, hi, nullptr, s_k, s_v,
+                                                                                   (uint16_t (*)[kBins])s_cnt, s_wave_sum, &s_flag);
                 }
+                if (through_memory) sort_segment_general(keys, values, alt_keys, alt_values, lo, hi, s_cnt, s_wave_sum, &s_flag);
             }
-        }
-        const uint32_t count = list_count[(kAllClasses ? 3 * kListShards : 0) + shard];
-        for (uint32_t i = blockIdx.x / kListShards; i < count; i += list_blocks / kListShards) {
-            const uint32_t v = list[(size_t)shard * list_cap + i];
-            sort_segment_general(keys, values, alt_keys, alt_values, seg_start[v], seg_start[v + 1], s_cnt, s_wave_sum, &s_flag);
         }
         return;
     }
@@ -1457,22 +1460,20 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         }
 #undef FGS_SEGMENT_CLASS
         // longer segments from their list, one workgroup per segment; behind them the shorter ones that were flagged
-        if (merged_tail || merged_large) {
-            const int smallest = merged_tail ? kCapSmall : kCapMedium;
-            const unsigned blocks = n > smallest ? list_grid((unsigned)(n / (smallest + 1) + 1), 256u) : 0u;
+        if (seg_start) {
+            const int smallest = merged_tail ? kCapSmall : merged_large ? kCapMedium : kCapLarge;
+            const unsigned blocks = n > smallest ? list_grid((unsigned)(n / (smallest + 1) + 1), n > kMergedLargeMax ? 2048u : 256u) : 0u;
             hipLaunchKernelGGL(segment_sort_general_kernel<true>, dim3(blocks + (ids + kWave - 1) / kWave),
                                dim3(kGeneralWaves * kWave), 0, st, ks, vs, alt_keys, alt_values, n, tile_mask, kCapLarge, ids,
                                (const int*)seg_start, (const uint32_t*)seg_flags,
                                (const uint32_t*)list_long, (const uint32_t*)seg_counts, cap_long, blocks,
                                (const uint32_t*)list_medium, cap_medium, (const uint32_t*)list_large, cap_large,
-                               merged_tail ? 1 : 2);
+                               merged_tail ? 1 : merged_large ? 2 : 3);
         } else {
-            const unsigned long_blocks = seg_start && n > kCapLarge ? list_grid((unsigned)(n / (kCapLarge + 1) + 1), 2048u) : 0u;
-            hipLaunchKernelGGL(segment_sort_general_kernel<false>, dim3(seg_start ? long_blocks + (ids + kWave - 1) / kWave : ids),
+            hipLaunchKernelGGL(segment_sort_general_kernel<false>, dim3(ids),
                                dim3(kGeneralWaves * kWave), 0, st, ks, vs, alt_keys, alt_values, n, tile_mask, kCapLarge, ids,
                                (const int*)seg_start, (const uint32_t*)seg_flags,
-                               (const uint32_t*)list_long, (const uint32_t*)(seg_counts + 3 * kListShards), cap_long, long_blocks,
-                               no_list, 0u, no_list, 0u, 0);
+                               no_list, no_list, 0u, 0u, no_list, 0u, no_list, 0u, 0);
         }
     }
     return check_hip(hipGetLastError(), "sort launch");
