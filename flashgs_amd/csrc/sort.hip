@@ -520,7 +520,7 @@ __global__ __launch_bounds__(kSortBlock) void scatter_kernel(
 constexpr int kCapTiny = 512, kCapSmall = 1024, kCapMedium = 4096, kCapLarge = 8192;
 constexpr int kMergedLargeMax = 1 << 24;     // up to this many pairs the last launch also takes the class of 4097 .. 8192 pairs
 constexpr int kMergedTailMax = 1 << 19;      // up to this many pairs the last launch also takes the classes of 1025 .. 8192 pairs
-constexpr uint32_t kOneLaunchIds = 32768;    // up to this many tile ids one launch sorts every segment of up to kCapSmall pairs
+constexpr uint32_t kOneLaunchIds = 262144;   // up to this many tile ids one launch sorts every segment of up to kCapSmall pairs
 
 // First index in [0, n) whose tile field is >= v (n if none), found by the whole wave probing 64
 // evenly spaced positions per step.  `keys` is ordered by tile field.  All lanes return the same.
@@ -1422,10 +1422,13 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         // Up to 512 pairs: one wave, bitonic network in registers; one tile id per wave (neighbouring
         // tiles tend to be equally busy, so a wave that took several of them would become the tail
         // of the launch).  With a table the launch also lists the longer segments.
-        // A frame of few tiles has few segments of 513..1024 pairs, about one wave per SIMD, and a
-        // launch of their own lasts as long as one such sort: there the first launch takes them
-        // too, with 16 register slots (1080p: -15 us, 4K: -8 us; at 8K +40 us, because the launch
-        // over 131 072 ids, most of them under 128 pairs, then runs at fewer waves per SIMD).
+        // Up to kOneLaunchIds tile ids the first launch takes the segments of 513..1024 pairs too,
+        // with 16 register slots: on a frame of few tiles there are few of them, about one wave per
+        // SIMD, and a launch of their own lasts as long as one such sort (1080p: -15 us, 4K: -8 us).
+        // While the 16-slot code needed 145 registers, the launch over the 131 072 ids of an 8K
+        // frame, most of them under 128 pairs, lost more to the three waves per SIMD than the
+        // second launch cost (+40 us); at 75 registers it wins there as well (-12 us, and -0.28 ms
+        // on the 8K frame of 109M pairs).
         if (one_wave_launch)
             hipLaunchKernelGGL((segment_sort_wave_kernel<kCapSmall / kWave, 1>), dim3(ids), dim3(kWave),
                                0, st, ks, vs, n, tile_mask, 1, ids, (const int*)seg_start, seg_flags,

@@ -906,7 +906,7 @@ def _sort_case(tile, depth_bits, W, H, junk=None, seed=0, ascending=False):
 
 
 @pytest.mark.parametrize("dense", [False, True])
-@pytest.mark.parametrize("seg", [1500, 3000, 5000, 8000, 8192, 8193, 40000])
+@pytest.mark.parametrize("seg", [1500, 3000, 5000, 8000, 8192, 8193, 12000, 16384, 16385, 40000])
 def test_sort_segment_size_classes(seg, dense):
     """Tiles holding 1500 ... 40000 pairs: every size class of the per-tile depth sort, with many
     equal depths and with depths that agree in whole bytes (skipped passes); on a frame of many
