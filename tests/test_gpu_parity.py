@@ -399,8 +399,9 @@ def test_rasterizer_relaunches_once_after_a_scan_that_gave_up():
 
 
 def test_preprocess_replayed_from_a_captured_graph():
-    """fgs_preprocess keeps no per-launch state on the host, so a captured launch can be replayed:
-    every replay (with eager launches of other sizes in between) gives the eager result."""
+    """The preprocess entry points keep no per-launch state on the host, so a captured launch
+    (here the one that also mirrors its count into pinned memory) can be replayed: every replay
+    (with eager launches of other sizes in between) gives the eager result."""
     import gpu_pipeline as gp
     import torch
     from flashgs_amd import cabi
@@ -417,6 +418,7 @@ def test_preprocess_replayed_from_a_captured_graph():
     keys = torch.zeros(cap, device=gp.DEV, dtype=torch.int64)
     values = torch.zeros(cap, device=gp.DEV, dtype=torch.int32)
     off = torch.zeros(1, device=gp.DEV, dtype=torch.int32)
+    word = torch.full((1,), cabi.COUNT_PENDING, dtype=torch.int32).pin_memory()     # the captured launch also mirrors its count
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     graph = torch.cuda.CUDAGraph()
@@ -425,11 +427,14 @@ def test_preprocess_replayed_from_a_captured_graph():
         cabi.preprocess(n, sd.position.data_ptr(), sd.shs.data_ptr(), sd.opacity.data_ptr(), sd.cov3d.data_ptr(),
                         cam.width, cam.height, 16, 16, cam.position, cam.rotation, cam.focal_x, cam.focal_y,
                         cam.zFar, cam.zNear, xy.data_ptr(), rgb.data_ptr(), co.data_ptr(),
-                        keys.data_ptr(), values.data_ptr(), off.data_ptr(), cap, torch.cuda.current_stream().cuda_stream)
+                        keys.data_ptr(), values.data_ptr(), off.data_ptr(), cap, torch.cuda.current_stream().cuda_stream,
+                        count_mirror=word.data_ptr())
     small = gp.SceneOnDevice(scenes.config0(n=3000))
     for replay in range(4):
         keys.zero_(); values.zero_()
+        word[0] = cabi.COUNT_PENDING
         graph.replay()
+        assert cabi.wait_count(word.data_ptr()) == K, "replay %d" % replay
         torch.cuda.synchronize()
         assert int(off.cpu()[0]) == K, "replay %d" % replay
         assert np.array_equal(gp.u64(keys)[:K], ref_keys), "replay %d" % replay
