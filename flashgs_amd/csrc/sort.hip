@@ -1411,6 +1411,8 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
         uint32_t* list_long = list_large + (size_t)kListShards * cap_large;
         const uint32_t* no_list = nullptr;
         // grids of the list-driven launches: a multiple of kListShards, enough for every listed segment
+        // (the limits are several times what is resident at once: a workgroup takes every
+        // (grid / kListShards)-th segment of its shard, and the shards are not equally long)
         auto list_grid = [](unsigned most, unsigned limit) {
             const unsigned g = most < limit ? most : limit;
             return (g + kListShards - 1) / kListShards * kListShards;
@@ -1450,10 +1452,10 @@ extern "C" int fgs_sort_gaussian(int num_rendered,
                                    dim3(kWave), 0, st, ks, vs, (const int*)seg_start, seg_flags,
                                    (const uint32_t*)list_small, (const uint32_t*)seg_counts, cap_small);
             if (n > kCapSmall && !merged_tail) {
-                FGS_SEGMENT_CLASS(8, kCapMedium, 64, kCapSmall, list_grid((unsigned)(n / (kCapSmall + 1) + 1), 1024u),
+                FGS_SEGMENT_CLASS(8, kCapMedium, 64, kCapSmall, list_grid((unsigned)(n / (kCapSmall + 1) + 1), 4096u),
                                   list_medium, seg_counts + kListShards, cap_medium);
                 if (n > kCapMedium && !merged_large)
-                    FGS_SEGMENT_CLASS(16, kCapLarge, 64, kCapMedium, list_grid((unsigned)(n / (kCapMedium + 1) + 1), 256u),
+                    FGS_SEGMENT_CLASS(16, kCapLarge, 64, kCapMedium, list_grid((unsigned)(n / (kCapMedium + 1) + 1), 1024u),
                                       list_large, seg_counts + 2 * kListShards, cap_large);
             }
         } else {
