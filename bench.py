@@ -41,7 +41,7 @@ EXEC_SLOTS_PER_EVAL = 8.1        # non-transcendental VALU instructions the fp32
                                  # profiles/frame_cfg2_3M_4K_sq_counters.txt): 2 for the exponent from its tables, alpha*T, T -=,
                                  # 3 colour FMAs, 1.1 for staging, stop tests and loop; the v_exp_f32 issues beside them
 ATTAINED_FMA_LANE_OPS = 38.05e12 # v_fma_f32 lane-operations/s measured on this part without packed math (bench.py --calibrate)
-CAPACITY = {0: 1 << 20, 1: 1 << 22, 2: 1 << 24, 3: 1 << 25, 4: 1 << 25, 5: 1 << 27}
+CAPACITY = {0: 1 << 20, 1: 1 << 22, 2: 1 << 24, 3: 1 << 25, 4: 1 << 25, 5: 1 << 27, 6: 1 << 25}
 FAST_MODE_DTYPE = "f32 (colour sums: f16 operands on the matrix unit, fp32 products and sums)"
 
 
@@ -53,7 +53,8 @@ def parse():
                     help="untimed frames first; the clocks of an idle GPU take about 50 frames of the 4K workload to settle")
     ap.add_argument("--config", type=int, default=2,
                     help="index into BASELINE.json configs (default: the 4K / 3M headline); 5 = the 8K scene with every "
-                         "splat five times as large (more than 100M pairs)")
+                         "splat five times as large (more than 100M pairs); 6 = the orbit scene with its anisotropic "
+                         "tenth stored last")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-reps", type=int, default=3)
     ap.add_argument("--headline-only", action="store_true", help="skip the other configurations (field \"configs\")")
@@ -395,8 +396,8 @@ def main():
 
     size = None
     if args.size:
-        if args.config != 4:
-            sys.exit("bench.py: --size applies to the trajectory workload (--config 4) only")
+        if args.config not in (4, 6):
+            sys.exit("bench.py: --size applies to the trajectory workload (--config 4 or 6) only")
         size = tuple(int(v) for v in args.size.lower().split("x"))
     with_cpu = not args.no_cpu_baseline
 
@@ -451,7 +452,7 @@ def main():
     if not args.headline_only:
         others = {}
         big = None          # the 8M scene, generated once for the 8K configuration and its dense variant
-        for config, sz in ((0, None), (1, None), (2, None), (3, None), (5, None), (4, None), (4, (3840, 2160))):
+        for config, sz in ((0, None), (1, None), (2, None), (3, None), (5, None), (4, None), (4, (3840, 2160)), (6, (3840, 2160))):
             if config == args.config and sz == size:
                 continue
             rep, fr_o = run_config(mods, config, sz, args.other_steps, min(args.warmup, 3), 1, with_cpu, False,

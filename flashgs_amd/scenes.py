@@ -214,9 +214,12 @@ def config3_dense(n=8_000_000, base=None):
                  list(sc.cameras))
 
 
-def config4(n=2_000_000, width=1920, height=1080, n_poses=60):
+def config4(n=2_000_000, width=1920, height=1080, n_poses=60, aniso_last=False):
     """Orbit of 60 poses (radius 30, height 5, 6 degree steps) around the cluster scene; 10 % of
-    the Gaussians are 100:1 anisotropic and lie within 1 unit of the camera path."""
+    the Gaussians are 100:1 anisotropic and lie within 1 unit of the camera path.  They are a
+    random subset of the indices; with `aniso_last` they are stored as the last tenth of the
+    scene instead (name ..._needles_last), which is the worst case for a preprocess that hands
+    out key slots in index order: the workgroups that hold them then all run at the end."""
     rng = np.random.default_rng(4)
     n_aniso = n // 10
     n_reg = n - n_aniso
@@ -231,15 +234,24 @@ def config4(n=2_000_000, width=1920, height=1080, n_poses=60):
     a_ls[:, 0] += math.log(100.0)                 # one long axis: ratio 100:1
     means = np.concatenate([means, a_means], axis=0)
     log_scales = np.concatenate([log_scales, a_ls], axis=0)
+    if not aniso_last:
+        place = np.random.default_rng(44).permutation(n)       # a generator of its own: everything else is drawn as before
+        means, log_scales = means[place], log_scales[place]
     cams = []
     for k in range(n_poses):
         a = math.radians(6.0 * k)
         pos = np.array([30.0 * math.sin(a), 5.0, -30.0 * math.cos(a)])
         cams.append(look_at(pos, [0, 0, 0], width, height, 60.0))
-    return _finish("cfg4_2M_orbit_%dx%d" % (width, height), rng, means, log_scales, 0.0, 2.0, cams)
+    name = "cfg4_2M_orbit_%dx%d%s" % (width, height, "_needles_last" if aniso_last else "")
+    return _finish(name, rng, means, log_scales, 0.0, 2.0, cams)
 
 
-CONFIGS = {0: config0, 1: config1, 2: config2, 3: config3, 4: config4, 5: config3_dense}
+def config4_needles_last(**kw):
+    """The orbit scene with its anisotropic tenth stored last (see config4)."""
+    return config4(aniso_last=True, **kw)
+
+
+CONFIGS = {0: config0, 1: config1, 2: config2, 3: config3, 4: config4, 5: config3_dense, 6: config4_needles_last}
 
 
 def make(config, **kw):

@@ -15,7 +15,7 @@ IMG_U8_FRACTION = 0.01
 # With the colour sums on the matrix unit (opt-in) weights and colours are rounded to f16 (products
 # and sums in fp32): a pixel's colour is within 2^-10 of itself of the oracle's, which moves a few
 # more of those 8-bit values.
-IMG_U8_FRACTION_F16 = 0.02
+IMG_U8_FRACTION_F16 = 0.03     # a guard against a systematic shift only: the bound proper is the per-pixel one (2^-10 of the colour)
 
 
 def _oracle_frame(oracle, sc, cam, capacity, block=(16, 16), bg=(0, 0, 0), sentinel=0.0):
@@ -219,9 +219,12 @@ def test_degenerate_inputs_match_the_oracle(oracle):
     assert np.array_equal(rg.cpu().numpy(), oracle.ranges(K, oks, rg.shape[0]))
 
 
-def test_anisotropic_splats_near_camera(oracle):
-    """Needle-shaped splats close to the camera: the exact ellipse test rejects most candidates."""
-    sc = scenes.config4(n=60_000, width=1280, height=720, n_poses=3)
+@pytest.mark.parametrize("aniso_last", [False, True])
+def test_anisotropic_splats_near_camera(oracle, aniso_last):
+    """Needle-shaped splats close to the camera: the exact ellipse test rejects most candidates.
+    As a random subset of the scene and stored as its last tenth (then the last workgroups hold
+    nothing else and their lists of big rectangles run full)."""
+    sc = scenes.config4(n=60_000, width=1280, height=720, n_poses=3, aniso_last=aniso_last)
     for cam in sc.cameras:
         ref = _check_frame(oracle, sc, cam, 1 << 22)
         assert ref["K"] < ref["pre"]["counts"]["candidates"]
@@ -847,6 +850,15 @@ def test_orbit_config_at_4k(oracle):
     candidate rectangles of thousands of tiles, which the workgroup tests from column and row spans."""
     sc = scenes.make(4, width=3840, height=2160)
     for cam in sc.cameras[::6] + [sc.cameras[-1]]:
+        ref = _check_frame(oracle, sc, cam, 1 << 25)
+        assert ref["pre"]["counts"]["candidates"] > 5 * ref["K"]
+
+
+def test_orbit_config_at_4k_with_the_needles_stored_last(oracle):
+    """The same scene with its anisotropic tenth stored last: the last 780 workgroups hold nothing
+    but needles, up to the 27 listed rectangles each and more.  Three poses."""
+    sc = scenes.make(6, width=3840, height=2160)
+    for cam in sc.cameras[::25]:
         ref = _check_frame(oracle, sc, cam, 1 << 25)
         assert ref["pre"]["counts"]["candidates"] > 5 * ref["K"]
 
