@@ -1145,6 +1145,7 @@ int preprocess_impl(bool allocate, const char* who, int P,
             return fail(FGS_E_INVALID, "%s: count_mirror must be pinned host memory (hipHostMalloc)", who);
         }
         mirror_on_device = (int*)mapped;
+        *(volatile int*)count_mirror = FGS_COUNT_PENDING;      // whatever an earlier frame left there is not this launch's count
     }
     if (P == 0) {
         if (mirror_on_device) {

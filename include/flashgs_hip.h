@@ -98,7 +98,8 @@ int fgs_preprocess_static(int P,
  * No counterpart in the reference, whose caller reads the pair count back with a blocking copy
  * (example.py:79).  fgs_preprocess that also stores the pair count into *count_mirror, a word of
  * pinned host memory (hipHostMalloc; anything else returns FGS_E_INVALID), for a host that polls
- * it instead (fgs_wait_count): the caller sets *count_mirror = FGS_COUNT_PENDING before the call.
+ * it instead (fgs_wait_count).  The call itself writes FGS_COUNT_PENDING into *count_mirror before
+ * it launches; a captured launch that is replayed does not, there the caller does before every replay.
  * The count arrives as soon as the launch knows it, which is while it is still writing keys: the
  * caller can enqueue fgs_sort_gaussian on the same stream at once, stream order does the rest.
  * A launch that gives up (see fgs_preprocess) stores INT_MIN; if only one workgroup's wait gives up

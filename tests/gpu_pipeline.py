@@ -37,7 +37,7 @@ def preprocess(sd, cam, capacity, block=(16, 16), sentinel=None, start_offset=0,
     keys = torch.zeros(capacity + pad, device=DEV, dtype=torch.int64)
     values = torch.zeros(capacity + pad, device=DEV, dtype=torch.int32)
     curr_offset = torch.full((1,), start_offset, device=DEV, dtype=torch.int32)
-    word = torch.full((1,), cabi.COUNT_PENDING, dtype=torch.int32).pin_memory() if mirror else None
+    word = torch.full((1,), 777, dtype=torch.int32).pin_memory() if mirror else None     # stale: the call marks it pending itself
     cabi.preprocess(n, sd.position.data_ptr(), sd.shs.data_ptr(), sd.opacity.data_ptr(), sd.cov3d.data_ptr(),
                     cam.width, cam.height, block[0], block[1], cam.position, cam.rotation,
                     cam.focal_x, cam.focal_y, cam.zFar, cam.zNear,
