@@ -146,6 +146,21 @@ void check_arguments()
     expect(fgs_set_colour_sums(FGS_COLOUR_SUMS_FP32) == FGS_COLOUR_SUMS_FP32, "the default colour-sum mode is fp32");
     expect(std::strcmp(fgs_blend_kernel_name(8, 8, 64, 64, 0), "") == 0, "no kernel name for an unsupported tile");
     expect(fgs_abi_version() == FGS_ABI_VERSION, "ABI version of header and library agree");
+    {
+        // the host-side poll for the mirrored pair count: finds what is there, says so when nothing comes
+        int word = 4711, got = 0;
+        expect(fgs_wait_count(&word, 1.0, &got) == FGS_OK && got == 4711, "a count that is there is returned");
+        word = -2147483647 - 1;
+        expect(fgs_wait_count(&word, 1.0, &got) == FGS_OK && got == word, "a negative count is a count");
+        word = FGS_COUNT_PENDING;
+        expect(fgs_wait_count(&word, 0.01, &got) == FGS_E_TIMEOUT && std::strlen(fgs_last_error()) > 0, "no count within the time given");
+        refused(fgs_wait_count(nullptr, 1.0, &got), "null count word");
+        refused(fgs_wait_count(&word, 1.0, nullptr), "null result");
+        refused(fgs_preprocess_mirrored(16, f, f, f, f, 64, 64, 16, 16, pos, rot, 1, 1, 100, 0.01f, f, f, f, k, v, i32, 16, nullptr, nullptr),
+                "null count mirror");
+        refused(fgs_preprocess_mirrored(-1, f, f, f, f, 64, 64, 16, 16, pos, rot, 1, 1, 100, 0.01f, f, f, f, k, v, i32, 16, &word, nullptr),
+                "negative P with a count mirror");
+    }
 }
 
 void check_host_arithmetic()
