@@ -19,7 +19,8 @@ operands) is reported beside it as ``fast_mode_*``.  ``roofline`` describes the 
 ``stages`` every stage with its algorithmic bytes against the 8 TB/s HBM peak, ``cpu_baseline`` the
 same frame computed by the multithreaded CPU oracle on this machine's host cores,
 ``ops_surface_ms_per_frame`` the same frame through ``flash_gaussian_splatting.ops`` the way
-``example.py:130-141`` times it, and ``configs`` the same figures for every other benchmark
+``example.py:130-141`` times it (``ops_surface_batch_ms_per_frame``: as one batch through
+``BatchRasterizer``, two frames in flight; ``two_frames_in_flight_*``: the same through the C ABI), and ``configs`` the same figures for every other benchmark
 configuration (the 60-pose orbit at both frame sizes with per-frame p50 / p99).
 """
 import argparse
@@ -199,6 +200,49 @@ class Frame:
             "position", "shs", "opacity", "cov3d", "points_xy", "rgb_depth", "conic_opacity", "keys_u", "vals_u",
             "keys_s", "vals_s", "sort_space", "ranges", "curr_offset", "out_color")}
 
+    def twin(self):
+        """A second set of work buffers and output image for the same scene (the scene tensors are shared)."""
+        import copy
+        torch, cabi = self.torch, self.cabi
+        t = copy.copy(self)
+        dev = self.position.device
+        for name in ("points_xy", "rgb_depth", "conic_opacity", "keys_u", "vals_u", "keys_s", "vals_s", "sort_space", "ranges",
+                     "curr_offset", "out_color"):
+            setattr(t, name, torch.zeros_like(getattr(self, name)))
+        t.offset_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        t.count_mirror = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        t.count_word = t.count_mirror.numpy()
+        t.P = {k: getattr(t, k).data_ptr() for k in self.P}
+        return t
+
+    def in_flight(self, cams, steps, warmup, sets=2):
+        """ms per frame with `sets` frames in flight: every set of work buffers has a stream of its own and
+        the frames go to the sets in turn, so that one frame's blend (bound by instruction issue) runs beside
+        the next frame's preprocess and sort (bound by memory).  Frame i + sets waits for frame i's image."""
+        torch = self.torch
+        frames = [self] + [self.twin() for _ in range(sets - 1)]
+        streams = [torch.cuda.Stream() for _ in frames]
+        saved = self.stream
+        for f, s in zip(frames, streams):
+            f.stream = s.cuda_stream
+
+        def run(n):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(n):
+                j = i % sets
+                with torch.cuda.stream(streams[j]):
+                    frames[j].frame(cams[i % len(cams)])
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) * 1e3 / n
+        try:
+            run(max(warmup, sets))
+            ms = run(steps)
+            same = all(bool(torch.equal(frames[0].out_color, f.out_color)) for f in frames[1:]) if len(cams) == 1 else None
+        finally:
+            self.stream = saved
+        return ms, same
+
     def frame(self, c, ev=None, flags=None):
         """One frame; `flags` (cabi.BLEND_*) chooses the blend's colour-sum mode for this call, None = the library default."""
         cabi, P, W, H, st = self.cabi, self.P, self.W, self.H, self.stream
@@ -332,7 +376,21 @@ def ops_surface_ms(torch, np, fr, steps):
     torch.cuda.synchronize()
     same = bool(torch.equal(img, fr.out_color))
     del rast
-    return round(ms, 4), same
+    # the same frames as one batch through BatchRasterizer: two frames in flight, every image kept
+    from flashgs_amd.rasterizer import BatchRasterizer
+    frames = min(steps, 64)
+    batch = BatchRasterizer(scene, fr.capacity, fr.tiles, frames_in_flight=2)
+    out = batch.render(scene, [cam] * frames, bg)
+    batch.render(scene, [cam] * frames, bg, out=out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(2):
+        batch.render(scene, [cam] * frames, bg, out=out)
+    torch.cuda.synchronize()
+    batch_ms = (time.perf_counter() - t0) * 1e3 / (2 * frames)
+    same = same and bool(torch.equal(out[0], fr.out_color)) and bool(torch.equal(out[-1], fr.out_color))
+    del batch, out
+    return round(ms, 4), same, round(batch_ms, 4)
 
 
 def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops, base=None):
@@ -346,6 +404,8 @@ def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops, 
     fr.blocking_readback = True
     blocking_ms, _, _, _ = fr.timed(fr.cams[:1], max(5, steps // 2), 2, False)
     fr.blocking_readback = False
+    # ... and with two frames in flight, each on a stream and a set of work buffers of its own
+    flight_ms, flight_same = fr.in_flight(fr.cams[:1], steps, min(warmup, 20))
     cpu, counts, walked = (None, None, None)
     if with_cpu:
         cpu, counts, walked = cpu_baseline(fr.sc, fr.cams[0], fr.capacity, cpu_reps)
@@ -356,6 +416,11 @@ def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops, 
                pair_count="stored into pinned host memory by the launch as soon as it is known and polled there "
                           "(fgs_preprocess_mirrored / fgs_wait_count)",
                blocking_readback_ms_per_frame=round(blocking_ms, 4),
+               two_frames_in_flight=dict(ms_per_frame=round(flight_ms, 4), fps=round(1000.0 / flight_ms, 2),
+                                         images_identical=flight_same,
+                                         what="the same frames sent in turn to two streams, each with work buffers and "
+                                              "an image of its own: one frame's blend runs beside the next frame's "
+                                              "preprocess and sort"),
                stage_timing="a second pass over the same steps with a HIP event in front of every stage",
                ms_per_frame_with_stage_events=round(instrumented_ms, 4),
                fast_mode=dict(dtype=FAST_MODE_DTYPE, ms_per_frame=round(fast_ms, 4), fps=round(1000.0 / fast_ms, 2),
@@ -371,8 +436,12 @@ def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops, 
                                  frame_ms_p50=round(frame_ms[len(frame_ms) // 2], 4),
                                  frame_ms_p99=round(frame_ms[min(len(frame_ms) - 1, int(0.99 * len(frame_ms)))], 4),
                                  stages_ms_mean={k: round(v, 4) for k, v in traj_stage.items()})
+        # the whole orbit as a batch: the poses in turn on two streams, no synchronisation between frames
+        batch_ms, _ = fr.in_flight(fr.cams, 2 * len(fr.cams), len(fr.cams) // 2)
+        rep["trajectory"]["batch_two_frames_in_flight_ms_per_frame"] = round(batch_ms, 4)
     if with_ops:
-        rep["ops_surface_ms_per_frame"], rep["ops_surface_image_identical"] = ops_surface_ms(torch, np, fr, steps)
+        (rep["ops_surface_ms_per_frame"], rep["ops_surface_image_identical"],
+         rep["ops_surface_batch_ms_per_frame"]) = ops_surface_ms(torch, np, fr, steps)
     return rep, fr
 
 
@@ -422,13 +491,16 @@ def main():
                    "tile": "16x16", "sh_degree": 3, "pairs": head["pairs"], "poses": head["poses"],
                    "stages_ms": {k: v["ms"] for k, v in head["stages"].items()},
                    "fast_mode": head["fast_mode"],
-                   "blocking_readback_ms_per_frame": head["blocking_readback_ms_per_frame"]},
+                   "blocking_readback_ms_per_frame": head["blocking_readback_ms_per_frame"],
+                   "two_frames_in_flight": head["two_frames_in_flight"]},
         "target_fps": 400 if args.config == 2 else None,
         "fast_mode_ms_per_frame": head["fast_mode"]["ms_per_frame"],
         "fast_mode_fps": head["fast_mode"]["fps"],
         "fast_mode_dtype": FAST_MODE_DTYPE,
         "pair_count": head["pair_count"],
         "blocking_readback_ms_per_frame": head["blocking_readback_ms_per_frame"],
+        "two_frames_in_flight_ms_per_frame": head["two_frames_in_flight"]["ms_per_frame"],
+        "two_frames_in_flight_fps": head["two_frames_in_flight"]["fps"],
         "stage_timing": head["stage_timing"],
         "ms_per_frame_with_stage_events": head["ms_per_frame_with_stage_events"],
         "stages": head["stages"],
@@ -436,6 +508,7 @@ def main():
         "cpu_baseline": head["cpu_baseline"],
         "ops_surface_ms_per_frame": head["ops_surface_ms_per_frame"],
         "ops_surface_image_identical": head["ops_surface_image_identical"],
+        "ops_surface_batch_ms_per_frame": head["ops_surface_batch_ms_per_frame"],
     }
     for k in ("n_pass", "visible", "walked"):
         if k in head:

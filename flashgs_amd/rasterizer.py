@@ -8,7 +8,8 @@ it is known (``ops.preprocess_mirrored`` / ``ops.wait_count``), instead of being
 a blocking read,
 the too-many-pairs condition raises a real exception (``example.py:82`` raises a string), a
 preprocess whose bounded waits gave up is launched once more after ``ops.reset_scan`` and raises
-``ScanGaveUp`` if that fails too, and the tile size is a constructor argument.
+``ScanGaveUp`` if that fails too, and the tile size is a constructor argument.  ``BatchRasterizer``
+renders a list of cameras with several frames in flight on streams of their own.
 """
 import json
 import os
@@ -125,7 +126,9 @@ class Rasterizer:
             self._out = torch.zeros((camera.height, camera.width, 3), device=device, dtype=torch.uint8)
         return self._out
 
-    def forward(self, scene, camera, bg_color):
+    def forward(self, scene, camera, bg_color, out=None):
+        """One frame.  The image is the rasterizer's own buffer (overwritten by the next frame) or,
+        if given, `out`: a contiguous uint8 (or int8) GPU tensor of height x width x 3."""
         o = ops()
         bx, by = self.tile
         tiles = ((camera.width + bx - 1) // bx) * ((camera.height + by - 1) // by)
@@ -161,12 +164,54 @@ class Rasterizer:
         o.sort_gaussian(num_rendered, camera.width, camera.height, bx, by, self.list_sorting_space,
                         self.gaussian_keys_unsorted, self.gaussian_values_unsorted,
                         self.gaussian_keys_sorted, self.gaussian_values_sorted)
-        out_color = self._image(camera, scene.device)
+        out_color = self._image(camera, scene.device) if out is None else out
         self._render(num_rendered, camera.width, camera.height,
                      self.points_xy, self.rgb_depth, self.conic_opacity,
                      self.gaussian_keys_sorted, self.gaussian_values_sorted,
                      self.ranges, bg_color, out_color)
         return out_color
+
+
+class BatchRasterizer:
+    """Renders a list of cameras with several frames in flight (no counterpart in the reference,
+    whose driver renders one frame after the other on one stream).
+
+    Every frame in flight has a `Rasterizer` - key, sort and attribute buffers - and a stream of
+    its own; the cameras go to them in turn.  The stages of one frame still follow each other,
+    but one frame's blend, which is bound by instruction issue, runs beside the next frame's
+    preprocess and sort, which are bound by memory, and a launch that leaves CUs idle (the tail
+    of a preprocess, the short kernels of a small frame) has the other frame's work to fill them.
+    The images are what `Rasterizer.forward` renders, frame by frame."""
+
+    def __init__(self, scene, MAX_NUM_RENDERED, MAX_NUM_TILES, frames_in_flight=2, tile=(16, 16)):
+        if frames_in_flight < 1:
+            raise ValueError("frames_in_flight must be at least 1")
+        self.rasterizers = [Rasterizer(scene, MAX_NUM_RENDERED, MAX_NUM_TILES, tile) for _ in range(frames_in_flight)]
+        self.streams = [torch.cuda.Stream(device=scene.device) for _ in range(frames_in_flight)]
+
+    def render(self, scene, cameras, bg_color, out=None):
+        """All `cameras` (of one image size); returns a uint8 tensor [len(cameras), height, width, 3]
+        (or fills `out`), ready for use on the current stream of the scene's device."""
+        cameras = list(cameras)
+        if not cameras:
+            return out
+        h, w = cameras[0].height, cameras[0].width
+        if any(c.height != h or c.width != w for c in cameras):
+            raise ValueError("the cameras of a batch must have one image size")
+        if out is None:
+            out = torch.empty((len(cameras), h, w, 3), device=scene.device, dtype=torch.uint8)
+        if tuple(out.shape) != (len(cameras), h, w, 3) or not out.is_contiguous():
+            raise ValueError("out must be a contiguous tensor of shape %r" % ((len(cameras), h, w, 3),))
+        caller = torch.cuda.current_stream(scene.device)
+        for s in self.streams:
+            s.wait_stream(caller)              # the scene and `out` as the caller's stream leaves them
+        for i, camera in enumerate(cameras):
+            j = i % len(self.streams)
+            with torch.cuda.stream(self.streams[j]):
+                self.rasterizers[j].forward(scene, camera, bg_color, out=out[i])
+        for s in self.streams:
+            caller.wait_stream(s)
+        return out
 
 
 def savePpm(image, path):

@@ -367,6 +367,30 @@ def test_scan_that_gives_up_reports_a_negative_count_until_reset():
             assert np.array_equal(gp.u32(again["values"])[:n], gp.u32(want["values"])[:n])
 
 
+@pytest.mark.parametrize("frames_in_flight", [1, 2, 3])
+def test_batch_rasterizer_renders_what_the_rasterizer_renders(frames_in_flight):
+    """BatchRasterizer: the poses of an orbit on two or three streams, each with buffers of its
+    own - the images are those of Rasterizer.forward, pose by pose, also when the batch is
+    rendered a second time into the same tensor."""
+    import gpu_pipeline as gp
+    import torch
+    from flashgs_amd.rasterizer import BatchRasterizer, Camera, Rasterizer, Scene
+    sc = scenes.config4(n=120_000, width=1280, height=720, n_poses=7)
+    scene = Scene(torch.device(gp.DEV)).from_arrays(sc.position, sc.shs, sc.opacity, sc.cov3d)
+    cams = [Camera.from_synthetic(c, i) for i, c in enumerate(sc.cameras)]
+    bg = torch.tensor([0.1, 0.2, 0.3])
+    one = Rasterizer(scene, 1 << 22, 1 << 14)
+    want = torch.stack([one.forward(scene, c, bg).clone() for c in cams])
+    batch = BatchRasterizer(scene, 1 << 22, 1 << 14, frames_in_flight=frames_in_flight)
+    got = batch.render(scene, cams, bg)
+    assert got.shape == want.shape and torch.equal(got, want)        # read on the current stream, no synchronisation here
+    again = batch.render(scene, cams[::-1], bg, out=got)
+    assert again is got and torch.equal(got, want.flip(0))
+    assert batch.render(scene, [], bg) is None
+    with pytest.raises(ValueError, match="one image size"):
+        batch.render(scene, [cams[0], Camera.from_synthetic(scenes.config1(n=10).cameras[0])], bg)
+
+
 def test_rasterizer_relaunches_once_after_a_scan_that_gave_up():
     """Rasterizer.forward clears the scan status and launches the frame once more when the pair
     count comes back negative; with the waits still failing it raises ScanGaveUp, not TooManyPairs."""
