@@ -59,6 +59,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-reps", type=int, default=3)
     ap.add_argument("--headline-only", action="store_true", help="skip the other configurations (field \"configs\")")
+    ap.add_argument("--sequential-only", action="store_true",
+                    help="skip the pass with two frames in flight (for kernel traces: launches that run beside another "
+                         "frame's kernels take longer and would blur the per-kernel averages)")
     ap.add_argument("--other-steps", type=int, default=20, help="timed frames per other configuration")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 256 MiB device-to-device copy, as the known-size reference for FETCH_SIZE / WRITE_SIZE")
@@ -393,7 +396,7 @@ def ops_surface_ms(torch, np, fr, steps):
     return round(ms, 4), same, round(batch_ms, 4)
 
 
-def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops, base=None):
+def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops, base=None, in_flight=True):
     torch, np, cabi, scenes = mods
     fr = Frame(torch, np, cabi, scenes, config, size, base)
     ms_per_step, stage_ms, _, K = fr.timed(fr.cams[:1], steps, warmup, False)
@@ -405,7 +408,7 @@ def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops, 
     blocking_ms, _, _, _ = fr.timed(fr.cams[:1], max(5, steps // 2), 2, False)
     fr.blocking_readback = False
     # ... and with two frames in flight, each on a stream and a set of work buffers of its own
-    flight_ms, flight_same = fr.in_flight(fr.cams[:1], steps, min(warmup, 20))
+    flight_ms, flight_same = fr.in_flight(fr.cams[:1], steps, min(warmup, 20)) if in_flight else (None, None)
     cpu, counts, walked = (None, None, None)
     if with_cpu:
         cpu, counts, walked = cpu_baseline(fr.sc, fr.cams[0], fr.capacity, cpu_reps)
@@ -416,11 +419,10 @@ def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops, 
                pair_count="stored into pinned host memory by the launch as soon as it is known and polled there "
                           "(fgs_preprocess_mirrored / fgs_wait_count)",
                blocking_readback_ms_per_frame=round(blocking_ms, 4),
-               two_frames_in_flight=dict(ms_per_frame=round(flight_ms, 4), fps=round(1000.0 / flight_ms, 2),
-                                         images_identical=flight_same,
-                                         what="the same frames sent in turn to two streams, each with work buffers and "
-                                              "an image of its own: one frame's blend runs beside the next frame's "
-                                              "preprocess and sort"),
+               two_frames_in_flight=None if flight_ms is None else dict(
+                   ms_per_frame=round(flight_ms, 4), fps=round(1000.0 / flight_ms, 2), images_identical=flight_same,
+                   what="the same frames sent in turn to two streams, each with work buffers and an image of its own: "
+                        "one frame's blend runs beside the next frame's preprocess and sort"),
                stage_timing="a second pass over the same steps with a HIP event in front of every stage",
                ms_per_frame_with_stage_events=round(instrumented_ms, 4),
                fast_mode=dict(dtype=FAST_MODE_DTYPE, ms_per_frame=round(fast_ms, 4), fps=round(1000.0 / fast_ms, 2),
@@ -437,8 +439,9 @@ def run_config(mods, config, size, steps, warmup, cpu_reps, with_cpu, with_ops, 
                                  frame_ms_p99=round(frame_ms[min(len(frame_ms) - 1, int(0.99 * len(frame_ms)))], 4),
                                  stages_ms_mean={k: round(v, 4) for k, v in traj_stage.items()})
         # the whole orbit as a batch: the poses in turn on two streams, no synchronisation between frames
-        batch_ms, _ = fr.in_flight(fr.cams, 2 * len(fr.cams), len(fr.cams) // 2)
-        rep["trajectory"]["batch_two_frames_in_flight_ms_per_frame"] = round(batch_ms, 4)
+        if in_flight:
+            batch_ms, _ = fr.in_flight(fr.cams, 2 * len(fr.cams), len(fr.cams) // 2)
+            rep["trajectory"]["batch_two_frames_in_flight_ms_per_frame"] = round(batch_ms, 4)
     if with_ops:
         (rep["ops_surface_ms_per_frame"], rep["ops_surface_image_identical"],
          rep["ops_surface_batch_ms_per_frame"]) = ops_surface_ms(torch, np, fr, steps)
@@ -470,7 +473,8 @@ def main():
         size = tuple(int(v) for v in args.size.lower().split("x"))
     with_cpu = not args.no_cpu_baseline
 
-    head, fr = run_config(mods, args.config, size, args.steps, args.warmup, args.cpu_reps, with_cpu, True)
+    head, fr = run_config(mods, args.config, size, args.steps, args.warmup, args.cpu_reps, with_cpu, not args.sequential_only,
+                          in_flight=not args.sequential_only)
     if args.copy_calibration:
         src = torch.ones(64 << 20, device=dev, dtype=torch.float32)      # 256 MiB read + 256 MiB written
         dst = torch.empty_like(src)
@@ -499,16 +503,16 @@ def main():
         "fast_mode_dtype": FAST_MODE_DTYPE,
         "pair_count": head["pair_count"],
         "blocking_readback_ms_per_frame": head["blocking_readback_ms_per_frame"],
-        "two_frames_in_flight_ms_per_frame": head["two_frames_in_flight"]["ms_per_frame"],
-        "two_frames_in_flight_fps": head["two_frames_in_flight"]["fps"],
+        "two_frames_in_flight_ms_per_frame": (head["two_frames_in_flight"] or {}).get("ms_per_frame"),
+        "two_frames_in_flight_fps": (head["two_frames_in_flight"] or {}).get("fps"),
         "stage_timing": head["stage_timing"],
         "ms_per_frame_with_stage_events": head["ms_per_frame_with_stage_events"],
         "stages": head["stages"],
         "roofline": head["roofline"],
         "cpu_baseline": head["cpu_baseline"],
-        "ops_surface_ms_per_frame": head["ops_surface_ms_per_frame"],
-        "ops_surface_image_identical": head["ops_surface_image_identical"],
-        "ops_surface_batch_ms_per_frame": head["ops_surface_batch_ms_per_frame"],
+        "ops_surface_ms_per_frame": head.get("ops_surface_ms_per_frame"),
+        "ops_surface_image_identical": head.get("ops_surface_image_identical"),
+        "ops_surface_batch_ms_per_frame": head.get("ops_surface_batch_ms_per_frame"),
     }
     for k in ("n_pass", "visible", "walked"):
         if k in head:
