@@ -222,8 +222,11 @@ def savePpm(image, path):
         f.write(b'P6\n' + f'{image.size(1)} {image.size(0)}\n255\n'.encode() + image.numpy().tobytes())
 
 
-def render_scene(model_path, test_performance=False, device='cuda:0', MAX_NUM_RENDERED=2 ** 27, MAX_NUM_TILES=2 ** 20):
-    """example.py:105-144: render every camera of ``<model_path>/cameras.json`` to ``test_out/*.ppm``."""
+def render_scene(model_path, test_performance=False, device='cuda:0', MAX_NUM_RENDERED=2 ** 27, MAX_NUM_TILES=2 ** 20,
+                 frames_in_flight=1):
+    """example.py:105-144: render every camera of ``<model_path>/cameras.json`` to ``test_out/*.ppm``.
+    With ``frames_in_flight`` above 1 and ``test_performance`` the cameras of one image size are
+    also timed as a batch through ``BatchRasterizer``."""
     scene_path = os.path.join(model_path, "point_cloud", "iteration_30000", "point_cloud.ply")
     camera_path = os.path.join(model_path, "cameras.json")
     device = torch.device(device)
@@ -251,6 +254,19 @@ def render_scene(model_path, test_performance=False, device='cuda:0', MAX_NUM_RE
             print("elapsed time = %f ms" % ((t1 - t0) / n * 1000))
             print("fps = %f" % (n / (t1 - t0)))
         savePpm(image, os.path.join(image_dir, "%s.ppm" % camera.img_name))
+    if test_performance and frames_in_flight > 1 and cameras_json:
+        cameras = [Camera(c) for c in cameras_json]
+        cameras = [c for c in cameras if (c.width, c.height) == (cameras[0].width, cameras[0].height)]
+        del rasterizer
+        batch = BatchRasterizer(scene, MAX_NUM_RENDERED, MAX_NUM_TILES, frames_in_flight=frames_in_flight)
+        out = batch.render(scene, cameras, bg_color)
+        torch.cuda.synchronize()
+        t0 = time.time()
+        batch.render(scene, cameras, bg_color, out=out)
+        torch.cuda.synchronize()
+        t1 = time.time()
+        print("batch of %d cameras, %d frames in flight: elapsed time per frame = %f ms, fps = %f"
+              % (len(cameras), frames_in_flight, (t1 - t0) / len(cameras) * 1000, len(cameras) / (t1 - t0)))
 
 
 if __name__ == "__main__":

@@ -125,9 +125,10 @@ def test_render_scene_from_ply_and_cameras_json(oracle, tmp_path, capsys):
                          rotation=[[float(v) for v in row] for row in c.rotation], fx=c.focal_x, fy=c.focal_y))
     (model / "cameras.json").write_text(json.dumps(cams))
 
-    render_scene(str(model), test_performance=True, MAX_NUM_RENDERED=1 << 20, MAX_NUM_TILES=1 << 13)
+    render_scene(str(model), test_performance=True, MAX_NUM_RENDERED=1 << 20, MAX_NUM_TILES=1 << 13, frames_in_flight=2)
     out = capsys.readouterr().out
     assert "num_vertex = %d" % n in out and "fps = " in out
+    assert "batch of 1 cameras, 2 frames in flight" in out          # the second camera has another image size
 
     num, position, shs, opacity, cov3d = fgs.ops.loadPly(str(ply_dir / "point_cloud.ply"))
     assert num == n
