@@ -41,3 +41,25 @@ def test_pip_install_outside_the_repository(tmp_path):
     version, size = out[3].split()
     assert int(version) >= 1 and int(size) >= 12 << 20
     assert out[4] == str(target / "flashgs_amd" / "lib" / "libflashgs_hip.so")     # the one the extension mapped
+
+
+def test_the_product_never_reaches_the_cpu_oracle():
+    """The oracle is the checker of the tests: nothing that ships (the package, the headers,
+    ``setup.py``) imports, links, loads or starts it, and the built libraries do not depend on it."""
+    import re
+    reach = re.compile(r"\b(?:import\s+oracle|from\s+oracle|fgs_oracle|libfgs_oracle)\b|[\"'/]oracle/")
+    shipped = [os.path.join(ROOT, "setup.py")]
+    for top in ("flashgs_amd", "include"):
+        for folder, _, files in os.walk(os.path.join(ROOT, top)):
+            shipped += [os.path.join(folder, f) for f in files
+                        if f.endswith((".py", ".hip", ".cpp", ".h", ".hpp", ".inc"))]
+    assert len(shipped) > 10
+    for path in shipped:
+        with open(path, errors="replace") as fh:
+            hits = [line.strip() for line in fh if reach.search(line)]
+        assert not hits, (path, hits)
+    built = glob.glob(os.path.join(ROOT, "flashgs_amd", "lib", "*.so")) + glob.glob(os.path.join(ROOT, "flash_gaussian_splatting*.so"))
+    assert built, "nothing built: run __graft_entry__.build() first"
+    for lib in built:
+        needed = subprocess.check_output(["readelf", "-d", lib], timeout=60).decode()
+        assert "oracle" not in needed, lib
